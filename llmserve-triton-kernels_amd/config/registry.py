@@ -94,4 +94,10 @@ def read_config(model_dir: str | Path):
         raise FileNotFoundError(f"no config.json in {model_dir}")
     raw = json.loads(path.read_text())
     arch = architecture_of(raw)
-    return arch, arch.config_class.from_dict(raw), raw
+    config = arch.config_class.from_dict(raw)
+    if hasattr(config, "with_tensor_shapes"):
+        # a size that config.json leaves to a tensor's shape: the configuration takes it from the files' headers
+        from ..weights.loader import index_folder
+
+        config = config.with_tensor_shapes({name: shape for name, (_file, shape, _dtype) in index_folder(model_dir).items()})
+    return arch, config, raw

@@ -7,15 +7,20 @@
 //   conv_state    the ring takes the last taps - 1 projected rows of every request of the step (a kernel of its own,
 //                 because a token's write would race with its neighbours' reads; when every request brings one
 //                 token, conv_store writes the ring itself).
+//   norm_store    the same without a convolution, for queries and keys that are normed head by head: every head of q
+//                 and of k is divided by its root mean square over its dk numbers (eps inside the root) and multiplied by a
+//                 weight that all heads share; q is then multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) at
+//                 position p (every 0: no factor); all in 32-bit, rounded once, into the query rows and the cache slots.
 //   attend        one workgroup per new token, all heads.  Score heads s = h * maps + m (maps = 2: two score maps
 //                 per query head over the same values); s reads key head (h / (H / G)) * maps + m, values come from
 //                 value head h / (H / G).  A query at position i sees the key j <= i if
 //                     j >= chunk_start(i)  and  (i - j < window  or  j < keep_first)
-//                 (window 0: no window; chunk 0: no chunks).  score = q . k * scale - slope_h * (i - j); softmax over the
+//                 (window 0: no window; chunk 0: no chunks).  score = q . k * scale - slope_h * (i - j) + dist_bias[h, min(i - j,
+//                 dist_reach)] (a table per head over the distance, which stays at its last entry beyond dist_reach); softmax over the
 //                 visible keys in 32-bit, normalised before anything else happens to it; optionally the heads' weights
 //                 are mixed, w_h = sum_g talk[h, g] w_g; then the values.  maps = 2 ends with o = a_1 - lambda a_2;
 //                 head_norm divides a head's result by its root mean square (eps inside the root) and multiplies
-//                 by out_scale.
+//                 by out_scale.  With gate products z (32-bit) the result is multiplied by sigmoid(z[n, h * dv + d]).
 //
 // Keys are [pages, key heads, block, dk], values [pages, value heads, dv, block] (transposed inside a page).
 #include "common.h"
@@ -97,6 +102,55 @@ __global__ __launch_bounds__(AC_THREADS) void conv_state_kernel(
         ring[(size_t)(pos % (taps - 1)) * channels + c] = proj[(size_t)(first_row + pos - first_pos) * proj_stride + c];
 }
 
+// grid: (tokens, query heads + key heads + value heads); one wave per head
+template <typename T>
+__global__ __launch_bounds__(LLMS_WAVE) void norm_store_kernel(
+    T* __restrict__ q_out, int q_stride, const float* __restrict__ proj, int proj_stride, const float* __restrict__ q_norm,
+    const float* __restrict__ k_norm, float eps, float temp_coef, int temp_every, const int* __restrict__ positions,
+    const int* __restrict__ slots, T* __restrict__ k_pool, T* __restrict__ v_pool, int q_heads, int k_heads, int dk,
+    int v_heads, int dv, int block_size) {
+    const int n = blockIdx.x, lane = threadIdx.x;
+    int head = blockIdx.y;
+    const float* row = proj + (size_t)n * proj_stride;
+    if (head < q_heads + k_heads) {
+        const bool is_q = head < q_heads;
+        const float* src = row + (size_t)head * dk;  // (keys follow the queries)
+        const float* w = is_q ? q_norm : k_norm;
+        float mul = 1.f;
+        if (w) {
+            float ss = 0.f;
+            for (int d = lane; d < dk; d += LLMS_WAVE) ss = fmaf(src[d], src[d], ss);
+            mul = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
+        }
+        float factor = 1.f;
+        if (is_q && temp_every > 0) factor = 1.f + temp_coef * logf((float)((positions[n] + 1) / temp_every + 1));
+        T* dst;
+        if (is_q) {
+            dst = q_out + (size_t)n * q_stride + (size_t)head * dk;
+        } else {
+            if (!slots) return;
+            const int slot = slots[n];
+            if (slot < 0) return;
+            const int page = slot / block_size, off = slot % block_size;
+            dst = k_pool + (((size_t)page * k_heads + (head - q_heads)) * block_size + off) * dk;
+        }
+        for (int d = lane; d < dk; d += LLMS_WAVE) {
+            float x = src[d] * mul;
+            if (w) x *= w[d];
+            dst[d] = from_f32<T>(x * factor);
+        }
+        return;
+    }
+    head -= q_heads + k_heads;
+    if (!slots) return;
+    const int slot = slots[n];
+    if (slot < 0) return;
+    const int page = slot / block_size, off = slot % block_size;
+    const float* src = row + (size_t)(q_heads + k_heads) * dk + (size_t)head * dv;
+    for (int d = lane; d < dv; d += LLMS_WAVE)
+        v_pool[(((size_t)page * v_heads + head) * dv + d) * block_size + off] = from_f32<T>(src[d]);
+}
+
 // ------------------------------------------------------------------------------------------- attention
 struct ComposedArgs {
     int out_stride, q_stride, max_blocks;
@@ -104,6 +158,10 @@ struct ComposedArgs {
     int window, keep_first, chunk;
     float scale, lambda, eps, out_scale;
     int head_norm;
+    const float* dist_bias;  // [heads, dist_reach + 1], or null
+    int dist_reach;
+    const float* gate;  // 32-bit products [N, gate_stride], or null
+    int gate_stride;
 };
 
 template <typename T>
@@ -192,6 +250,7 @@ __global__ __launch_bounds__(AC_THREADS) void attend_composed_kernel(
                 const int page = table[j / bs], off = j % bs;
                 const T* kr = k_pool + (((size_t)page * (G * a.maps) + kh) * bs + off) * dk;
                 sc = dot_row<T>(qs + s * dk, kr, dk) - slope * (float)(p - j);
+                if (a.dist_bias) sc += a.dist_bias[(size_t)h * (a.dist_reach + 1) + min(p - j, a.dist_reach)];
             }
             const float m_new = fmaxf(m, wave_max(sc));
             const float e = v < n_vis ? expf(sc - m_new) : 0.f;
@@ -225,7 +284,8 @@ __global__ __launch_bounds__(AC_THREADS) void attend_composed_kernel(
             if (v < n_vis) {
                 const float slope = slopes ? slopes[h] : 0.f;
                 const T* kr = k_pool + (((size_t)page * (G * a.maps) + kh) * bs + off) * dk;
-                const float sc = dot_row<T>(qs + s * dk, kr, dk) - slope * (float)(p - j);
+                float sc = dot_row<T>(qs + s * dk, kr, dk) - slope * (float)(p - j);
+                if (a.dist_bias) sc += a.dist_bias[(size_t)h * (a.dist_reach + 1) + min(p - j, a.dist_reach)];
                 w = expf(sc - stat_m[s]) / stat_l[s];
             }
             prob[s * AC_TILE + lane] = w;
@@ -270,7 +330,9 @@ __global__ __launch_bounds__(AC_THREADS) void attend_composed_kernel(
         for (int d = lane; d < dv; d += LLMS_WAVE) {
             float o = acc_o[(h * a.maps) * dv + d];
             if (a.maps == 2) o -= a.lambda * acc_o[(h * 2 + 1) * dv + d];
-            orow[h * dv + d] = from_f32<T>(o * mul);
+            o *= mul;
+            if (a.gate) o /= 1.f + expf(-a.gate[(size_t)n * a.gate_stride + h * dv + d]);
+            orow[h * dv + d] = from_f32<T>(o);
         }
     }
 }
@@ -312,6 +374,28 @@ int llms_conv_store(int dtype, void* q_out, int q_stride, const float* proj, int
     LLMS_LAUNCH_CHECK();
 }
 
+int llms_norm_store(int dtype, void* q_out, int q_stride, const float* proj, int proj_stride, const float* q_norm,
+                    const float* k_norm, float eps, float temp_coef, int temp_every, const int* positions, const int* slots,
+                    void* k_pool, void* v_pool, int n_tokens, int q_heads, int k_heads, int dk, int v_heads, int dv,
+                    int block_size, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && q_heads > 0 && k_heads >= 0 && v_heads >= 0 && dk > 0 && dv > 0, "norm_store: sizes must be positive");
+    LLMS_REQUIRE(temp_every == 0 || positions, "norm_store: a factor by position needs the positions");
+    LLMS_REQUIRE(!slots || (k_pool && v_pool && block_size > 0), "norm_store: slots given without pools");
+    LLMS_REQUIRE(q_heads + k_heads + v_heads <= 65535, "norm_store: up to 65,535 heads in all");
+    dim3 grid(n_tokens, q_heads + k_heads + v_heads);
+    if (dtype == 0)
+        norm_store_kernel<float><<<grid, LLMS_WAVE, 0, stream>>>((float*)q_out, q_stride, proj, proj_stride, q_norm, k_norm, eps,
+                                                                 temp_coef, temp_every, positions, slots, (float*)k_pool,
+                                                                 (float*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size);
+    else if (dtype == 1)
+        norm_store_kernel<bf16><<<grid, LLMS_WAVE, 0, stream>>>((bf16*)q_out, q_stride, proj, proj_stride, q_norm, k_norm, eps,
+                                                                temp_coef, temp_every, positions, slots, (bf16*)k_pool,
+                                                                (bf16*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size);
+    else
+        LLMS_REQUIRE(false, "norm_store: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
 int llms_conv_state(float* state, size_t state_slot_stride, const int* state_slots, const float* proj, int proj_stride,
                     const int* cu_seqlens, const int* context_lens, int n_seqs, int taps, int channels,
                     hipStream_t stream) {
@@ -328,8 +412,9 @@ int llms_attend_composed(int dtype, void* out, int out_stride, const void* q, in
                          int kv_heads, int maps,
                          int dk, int dv, int block_size, int window, int keep_first, int chunk, float scale,
                          const float* slopes, const float* talk, float lambda, int head_norm, float eps, float out_scale,
-                         hipStream_t stream) {
+                         const float* dist_bias, int dist_reach, const float* gate, int gate_stride, hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && heads > 0 && kv_heads > 0 && dk > 0 && dv > 0, "attend_composed: sizes must be positive");
+    LLMS_REQUIRE(!dist_bias || dist_reach >= 0, "attend_composed: a distance table has at least one entry per head");
     LLMS_REQUIRE(heads % kv_heads == 0, "attend_composed: heads must be a multiple of kv_heads");
     LLMS_REQUIRE(maps == 1 || maps == 2, "attend_composed: one or two score maps");
     LLMS_REQUIRE(!(talk && maps != 1), "attend_composed: mixing heads' weights goes with one score map");
@@ -342,6 +427,7 @@ int llms_attend_composed(int dtype, void* out, int out_stride, const void* q, in
     a.heads = heads, a.kv_heads = kv_heads, a.maps = maps, a.dk = dk, a.dv = dv, a.block_size = block_size;
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
     a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
+    a.dist_bias = dist_bias, a.dist_reach = dist_reach, a.gate = gate, a.gate_stride = gate_stride;
     if (dtype == 0) {
         auto kernel = attend_composed_kernel<float>;
         if (lds > 48 * 1024)

@@ -5,7 +5,8 @@
 //                             its group and tile from tile_start[g] = tiles of all groups before g
 // Epilogues: plain; "paired" for a weight that stacks two projections a, b of a gated unit in blocks of 64 rows (32
 // rows of a, then the 32 rows of b of the same units, so that a thread or lane holds both of a unit):
-// out[m, u] = min(a, limit) * sigmoid(1.702 min(a, limit)) * (clamp(b, -limit, limit) + 1) for the `units` units;
+// out[m, u] = min(a, limit) * sigmoid(1.702 min(a, limit)) * (clamp(b, -limit, limit) + 1) for the `units` units
+// (unit 0), or a * sigmoid(a) * b (unit 1);
 // "gated": the result times sigmoid(z[m, g * z_gs + n]) with z in 32-bit.
 // Two kernels: 32-bit multiply-add (any sizes, float or bfloat16 operands, 32-bit products and sums) and bfloat16 on
 // the matrix cores (K and the strides of x in multiples of 8, 16-byte aligned operands).
@@ -19,9 +20,17 @@
 #define GG_PAIRED 1
 #define GG_GATED 2
 
+// which gated unit the paired epilogue forms
+#define GG_UNIT_CLAMPED 0
+#define GG_UNIT_SILU 1
+
 // (the operands of the gated unit are rounded as a stored activation would be)
 template <typename TOut>
-__device__ __forceinline__ float gated_unit(float a_sum, float b_sum, float limit) {
+__device__ __forceinline__ float gated_unit(float a_sum, float b_sum, float limit, int unit) {
+    if (unit == GG_UNIT_SILU) {
+        const float a = round_to<TOut>(a_sum), b = round_to<TOut>(b_sum);
+        return a / (1.f + expf(-a)) * b;
+    }
     const float a = fminf(round_to<TOut>(a_sum), limit);
     const float b = fminf(fmaxf(round_to<TOut>(b_sum), -limit), limit);
     return a / (1.f + expf(-1.702f * a)) * (b + 1.f);
@@ -31,7 +40,7 @@ template <typename TIn, typename TOut, int EPI>
 __global__ __launch_bounds__(256) void grouped_fma_kernel(
     TOut* __restrict__ out, long out_ld, long out_gs, const TIn* __restrict__ x, long x_ld, long x_gs,
     const TIn* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
-    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units) {
+    const float* __restrict__ z, long z_ld, long z_gs, float limit, int unit, int units) {
     __shared__ float As[GG_TK][GG_TM + 4];
     __shared__ float Ws[GG_TK][GG_TN + 4];
     const int tid = threadIdx.x;
@@ -89,7 +98,7 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
             for (int j = 0; j < 2; ++j) {
                 const int u = n0 / 2 + tn + j;
                 if (u >= units) continue;
-                og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][j], acc[i][j + 2], limit));
+                og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][j], acc[i][j + 2], limit, unit));
             }
         } else {
 #pragma unroll
@@ -107,10 +116,10 @@ __global__ __launch_bounds__(256) void grouped_fma_kernel(
 template <typename TIn, typename TOut>
 static int launch_fma(int epilogue, dim3 grid, hipStream_t stream, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                       long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
-                      long z_ld, long z_gs, float limit, int units) {
+                      long z_ld, long z_gs, float limit, int unit, int units) {
 #define GG_GO(EPI)                                                                                                          \
     grouped_fma_kernel<TIn, TOut, EPI><<<grid, 256, 0, stream>>>((TOut*)out, out_ld, out_gs, (const TIn*)x, x_ld, x_gs,      \
-                                                                 (const TIn*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units)
+                                                                 (const TIn*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, unit, units)
     if (epilogue == GG_PLAIN) GG_GO(GG_PLAIN);
     else if (epilogue == GG_PAIRED) GG_GO(GG_PAIRED);
     else GG_GO(GG_GATED);
@@ -140,7 +149,7 @@ template <typename TOut, int EPI>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(
     TOut* __restrict__ out, long out_ld, long out_gs, const bf16* __restrict__ x, long x_ld, long x_gs,
     const bf16* __restrict__ w, int M, int N, int K, int G, const int* __restrict__ seg, const int* __restrict__ tile_start,
-    const float* __restrict__ z, long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
+    const float* __restrict__ z, long z_ld, long z_gs, float limit, int unit, int units, int k_part, long part_stride) {
     extern __shared__ __attribute__((aligned(16))) uint16_t gm_lds[];
     uint16_t(*As)[GM_BM * GM_LD] = reinterpret_cast<uint16_t(*)[GM_BM * GM_LD]>(gm_lds);
     uint16_t(*Bs)[GM_BN * GM_LD] = reinterpret_cast<uint16_t(*)[GM_BN * GM_LD]>(gm_lds + 2 * GM_BM * GM_LD);
@@ -229,7 +238,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
             if (m >= row_end) continue;
             if (EPI == GG_PAIRED) {
                 const int u = (n0 + wn) / 2 + l32;
-                if (u < units) og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][0][r], acc[i][1][r], limit));
+                if (u < units) og[(size_t)m * out_ld + u] = from_f32<TOut>(gated_unit<TOut>(acc[i][0][r], acc[i][1][r], limit, unit));
             } else {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -247,12 +256,12 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
 template <typename TOut>
 static int launch_mfma(int epilogue, dim3 grid, hipStream_t stream, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                        long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, const float* z,
-                       long z_ld, long z_gs, float limit, int units, int k_part, long part_stride) {
+                       long z_ld, long z_gs, float limit, int unit, int units, int k_part, long part_stride) {
 #define GM_GO(EPI)                                                                                                          \
     LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)grouped_mfma_kernel<TOut, EPI>,                                         \
                                        hipFuncAttributeMaxDynamicSharedMemorySize, GM_LDS_BYTES));                          \
     grouped_mfma_kernel<TOut, EPI><<<grid, 256, GM_LDS_BYTES, stream>>>((TOut*)out, out_ld, out_gs, (const bf16*)x, x_ld, x_gs, \
-                                                             (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, units, \
+                                                             (const bf16*)w, M, N, K, G, seg, tile_start, z, z_ld, z_gs, limit, unit, units, \
                                                              k_part, part_stride)
     if (epilogue == GG_PLAIN) {
         GM_GO(GG_PLAIN);
@@ -272,7 +281,7 @@ extern "C" {
 // tile_start[G], which the host bounds by ceil(M / 64) + G).
 int llms_grouped_fma(int in_dtype, int out_dtype, int epilogue, void* out, long out_ld, long out_gs, const void* x, long x_ld,
                      long x_gs, const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start,
-                     int max_tiles, const float* z, long z_ld, long z_gs, float limit, int units, hipStream_t stream) {
+                     int max_tiles, const float* z, long z_ld, long z_gs, float limit, int unit, int units, hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, "grouped_fma: sizes must be positive");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "grouped_fma: epilogue 0 (plain), 1 (paired) or 2 (gated)");
     LLMS_REQUIRE(epilogue != GG_PAIRED || (N % 64 == 0 && units > 0 && units <= N / 2),
@@ -283,13 +292,13 @@ int llms_grouped_fma(int in_dtype, int out_dtype, int epilogue, void* out, long 
     LLMS_REQUIRE(grid.y > 0 && grid.y <= 65535 && grid.z <= 65535, "grouped_fma: too many rows or groups for one launch");
     if (in_dtype == 0 && out_dtype == 0)
         return launch_fma<float, float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start,
-                                        z, z_ld, z_gs, limit, units);
+                                        z, z_ld, z_gs, limit, unit, units);
     if (in_dtype == 1 && out_dtype == 1)
         return launch_fma<bf16, bf16>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z,
-                                      z_ld, z_gs, limit, units);
+                                      z_ld, z_gs, limit, unit, units);
     if (in_dtype == 1 && out_dtype == 0)
         return launch_fma<bf16, float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z,
-                                       z_ld, z_gs, limit, units);
+                                       z_ld, z_gs, limit, unit, units);
     LLMS_REQUIRE(false, "grouped_fma: unsupported dtype pair");
 }
 
@@ -298,7 +307,7 @@ int llms_grouped_fma(int in_dtype, int out_dtype, int epilogue, void* out, long 
 // leaving its sums at out + p * part_stride.
 int llms_grouped_mfma(int out_dtype, int epilogue, void* out, long out_ld, long out_gs, const void* x, long x_ld, long x_gs,
                       const void* w, int M, int N, int K, int G, const int* seg, const int* tile_start, int max_tiles,
-                      const float* z, long z_ld, long z_gs, float limit, int units, int k_parts, long part_stride,
+                      const float* z, long z_ld, long z_gs, float limit, int unit, int units, int k_parts, long part_stride,
                       hipStream_t stream) {
     LLMS_REQUIRE(M > 0 && N > 0 && K > 0 && G > 0, "grouped_mfma: sizes must be positive");
     LLMS_REQUIRE(epilogue >= 0 && epilogue <= 2, "grouped_mfma: epilogue 0 (plain), 1 (paired) or 2 (gated)");
@@ -316,10 +325,10 @@ int llms_grouped_mfma(int out_dtype, int epilogue, void* out, long out_ld, long 
     LLMS_REQUIRE(grid.y > 0 && grid.y <= 65535 && grid.z <= 65535, "grouped_mfma: too many rows or groups for one launch");
     if (out_dtype == 0)
         return launch_mfma<float>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
-                                  z_gs, limit, units, k_part, part_stride);
+                                  z_gs, limit, unit, units, k_part, part_stride);
     if (out_dtype == 1)
         return launch_mfma<bf16>(epilogue, grid, stream, out, out_ld, out_gs, x, x_ld, x_gs, w, M, N, K, G, seg, tile_start, z, z_ld,
-                                 z_gs, limit, units, k_part, part_stride);
+                                 z_gs, limit, unit, units, k_part, part_stride);
     LLMS_REQUIRE(false, "grouped_mfma: out_dtype must be 0 or 1");
 }
 

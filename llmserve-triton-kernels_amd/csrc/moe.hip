@@ -1,13 +1,16 @@
 // Routing for a feed-forward of many small experts, of which each token uses `top`.
-//   moe_router    z = W_router h in 32-bit, s = sigmoid(z), the `top` largest (the lower expert wins a tie), in descending order; weight = score or
-//                 score / sum of the chosen scores
+//   moe_router    z = W_router h in 32-bit, s = sigmoid(z) or softmax(z) over all experts, the `top` largest (the lower expert
+//                 wins a tie), in descending order; weight = score or score / (sum of the chosen scores + renorm_eps).
+//                 With `groups` > 1 the experts form that many equal groups of neighbours, a group's score is its largest
+//                 score, and only experts of the `keep` best groups (the lower group wins a tie) can be chosen
 //   moe_rank      for expert e: how many (token, choice) pairs chose it, and each such pair's rank among them in the
 //                 order of the pairs (so the sorted order is stable and the same whatever runs beside it)
 //   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of rows of all experts before e
 //   moe_scatter   rows sorted by expert: xs[seg[e] + rank] = weight * h[token] (the weight multiplies the expert's
-//                 input), rounded to T; place[pair] = that row
-//   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows (32-bit; a row may
-//                 arrive as partial sums over shares of the last product's K, added in the order of the shares)
+//                 input), rounded to T, or h[token] as it is where no weight is given; place[pair] = that row
+//   moe_combine   y[n] = sum over the token's choices, in their order, of the experts' results rows, each times its
+//                 weight where weights are given (32-bit; a row may arrive as partial sums over shares of the last
+//                 product's K, added in the order of the shares)
 // A pair is p = token * top + choice.
 #include "common.h"
 
@@ -17,8 +20,8 @@
 template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
     int* __restrict__ chosen, float* __restrict__ weight, const T* __restrict__ h, const T* __restrict__ w_router,
-    int hidden, int experts, int top, int renormalize) {
-    extern __shared__ float score[];  // experts
+    int hidden, int experts, int top, int renormalize, int softmax, int groups, int keep, float renorm_eps) {
+    extern __shared__ float score[];  // experts, then groups
     const int n = blockIdx.x, lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
     const T* row = h + (size_t)n * hidden;
     const bool vec = hidden % (16 / sizeof(T)) == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)w_router % 16) == 0;
@@ -51,10 +54,64 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
         dot = wave_sum(dot);
         // (a row that is not a number, as a padding row may be, gets a score like any other: every choice below must
         // name an expert that exists)
-        if (lane == 0) score[e] = dot == dot ? 1.f / (1.f + expf(-dot)) : 0.f;
+        if (lane == 0) score[e] = dot == dot ? (softmax ? dot : 1.f / (1.f + expf(-dot))) : 0.f;
     }
     __syncthreads();
     if (wave != 0) return;
+    if (softmax) {  // over all experts, in 32-bit: exp(z - max) / sum
+        float top_z = -INFINITY;
+        for (int e = lane; e < experts; e += LLMS_WAVE) top_z = fmaxf(top_z, score[e]);
+        top_z = wave_max(top_z);
+        float total = 0.f;
+        for (int e = lane; e < experts; e += LLMS_WAVE) {
+            const float w = expf(score[e] - top_z);
+            score[e] = w;
+            total += w;
+        }
+        total = wave_sum(total);
+        for (int e = lane; e < experts; e += LLMS_WAVE) score[e] = score[e] / total;
+        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_wave_barrier();
+    }
+    if (groups > 1) {  // experts outside the `keep` best groups are marked taken
+        float* best_of = score + experts;
+        const int per = experts / groups;
+        for (int g = lane; g < groups; g += LLMS_WAVE) {
+            float b = -1.f;
+            for (int e = g * per; e < (g + 1) * per; ++e) b = fmaxf(b, score[e]);
+            best_of[g] = b;
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_wave_barrier();
+        for (int k = 0; k < keep; ++k) {
+            float best = -1.f;
+            int at = 0x7fffffff;
+            for (int g = lane; g < groups; g += LLMS_WAVE) {
+                const float b = best_of[g];
+                if (b > best) {
+                    best = b;
+                    at = g;
+                }
+            }
+#pragma unroll
+            for (int o = LLMS_WAVE / 2; o > 0; o >>= 1) {
+                const float ob = __shfl_xor(best, o, LLMS_WAVE);
+                const int oa = __shfl_xor(at, o, LLMS_WAVE);
+                if (ob > best || (ob == best && oa < at)) {
+                    best = ob;
+                    at = oa;
+                }
+            }
+            at = min(at, groups - 1);
+            if (lane == 0) best_of[at] = -3.f;  // kept
+            __builtin_amdgcn_s_waitcnt(0);
+            __builtin_amdgcn_wave_barrier();
+        }
+        for (int e = lane; e < experts; e += LLMS_WAVE)
+            if (best_of[e / per] != -3.f) score[e] = -2.f;
+        __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_wave_barrier();
+    }
     float picked[MOE_MAX_TOP];
     int which[MOE_MAX_TOP];
     float sum = 0.f;
@@ -88,7 +145,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
     if (lane == 0)
         for (int k = 0; k < top; ++k) {
             chosen[(size_t)n * top + k] = which[k];
-            weight[(size_t)n * top + k] = renormalize ? picked[k] / sum : picked[k];
+            weight[(size_t)n * top + k] = renormalize ? picked[k] / (sum + renorm_eps) : picked[k];
         }
 }
 
@@ -144,17 +201,22 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_scatter_kernel(
     const float* __restrict__ weight, const int* __restrict__ rank, const int* __restrict__ seg, int hidden, int top) {
     const int p = blockIdx.x, n = p / top;
     const int dest = seg[chosen[p]] + rank[p];
-    const float wgt = weight[p];
     if (threadIdx.x == 0) place[p] = dest;
     const T* src = h + (size_t)n * hidden;
     T* dst = xs + (size_t)dest * hidden;
+    if (!weight) {
+        for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = src[c];
+        return;
+    }
+    const float wgt = weight[p];
     for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = from_f32<T>(wgt * to_f32(src[c]));
 }
 
 // grid: tokens.  rows [parts, pairs, hidden]: a choice's result may arrive as several partial sums
 __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ rows,
                                                                   const int* __restrict__ place, int hidden, int top,
-                                                                  int parts, long part_stride) {
+                                                                  int parts, long part_stride,
+                                                                  const float* __restrict__ weight) {
     const int n = blockIdx.x;
     if (hidden % 4 == 0 && part_stride % 4 == 0 && ((uintptr_t)rows % 16) == 0 && ((uintptr_t)y % 16) == 0) {
         // 16 bytes a thread and load, the loads of four summands in flight together
@@ -163,15 +225,24 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
             const int terms = top * parts;
             for (int t0 = 0; t0 < terms; t0 += 4) {
                 float4 part[4];
+                float wk[4];
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int t = t0 + u, k = t / parts, p = t - k * parts;
+                    wk[u] = (weight && t < terms) ? weight[(size_t)n * top + k] : 1.f;
                     part[u] = t < terms ? *reinterpret_cast<const float4*>(rows + (size_t)place[(size_t)n * top + k] * hidden +
                                                                            (size_t)p * part_stride + c)
                                         : make_float4(0.f, 0.f, 0.f, 0.f);
                 }
 #pragma unroll
-                for (int u = 0; u < 4; ++u) v.x += part[u].x, v.y += part[u].y, v.z += part[u].z, v.w += part[u].w;
+                for (int u = 0; u < 4; ++u) {
+                    if (weight) {
+                        v.x = fmaf(wk[u], part[u].x, v.x), v.y = fmaf(wk[u], part[u].y, v.y);
+                        v.z = fmaf(wk[u], part[u].z, v.z), v.w = fmaf(wk[u], part[u].w, v.w);
+                    } else {
+                        v.x += part[u].x, v.y += part[u].y, v.z += part[u].z, v.w += part[u].w;
+                    }
+                }
             }
             *reinterpret_cast<float4*>(y + (size_t)n * hidden + c) = v;
         }
@@ -181,7 +252,8 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
         float v = 0.f;
         for (int k = 0; k < top; ++k) {
             const float* row = rows + (size_t)place[(size_t)n * top + k] * hidden + c;
-            for (int p = 0; p < parts; ++p) v += row[(size_t)p * part_stride];
+            const float wk = weight ? weight[(size_t)n * top + k] : 1.f;
+            for (int p = 0; p < parts; ++p) v = weight ? fmaf(wk, row[(size_t)p * part_stride], v) : v + row[(size_t)p * part_stride];
         }
         y[(size_t)n * hidden + c] = v;
     }
@@ -190,18 +262,21 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
 extern "C" {
 
 int llms_moe_router(int dtype, int* chosen, float* weight, const void* h, const void* w_router, int n, int hidden, int experts,
-                    int top, int renormalize, hipStream_t stream) {
+                    int top, int renormalize, int softmax, int groups, int keep, float renorm_eps, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && hidden > 0 && experts > 0, "moe_router: sizes must be positive");
     LLMS_REQUIRE(top >= 1 && top <= MOE_MAX_TOP && top <= experts, "moe_router: 1 to 16 choices, no more than there are experts");
     LLMS_REQUIRE(experts <= 8192, "moe_router: up to 8,192 experts");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "moe_router: dtype must be 0 (float32) or 1 (bfloat16)");
-    const size_t lds = (size_t)experts * sizeof(float);
+    LLMS_REQUIRE(groups >= 1 && experts % groups == 0 && keep >= 1 && keep <= groups,
+                 "moe_router: the groups must share the experts out equally, and 1 to all of them are kept");
+    LLMS_REQUIRE(groups == 1 || top <= keep * (experts / groups), "moe_router: the kept groups hold fewer experts than are chosen");
+    const size_t lds = (size_t)(experts + groups) * sizeof(float);
     if (dtype == 0)
         moe_router_kernel<float><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const float*)h, (const float*)w_router, hidden,
-                                                                  experts, top, renormalize);
+                                                                  experts, top, renormalize, softmax, groups, keep, renorm_eps);
     else
         moe_router_kernel<bf16><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const bf16*)h, (const bf16*)w_router, hidden,
-                                                                 experts, top, renormalize);
+                                                                 experts, top, renormalize, softmax, groups, keep, renorm_eps);
     LLMS_LAUNCH_CHECK();
 }
 
@@ -228,9 +303,9 @@ int llms_moe_scatter(int dtype, void* xs, int* place, const void* h, const int* 
 }
 
 int llms_moe_combine(float* y, const float* rows, const int* place, int n, int hidden, int top, int parts, long part_stride,
-                     hipStream_t stream) {
+                     const float* weight, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && hidden > 0 && top > 0 && parts > 0, "moe_combine: sizes must be positive");
-    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top, parts, part_stride);
+    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top, parts, part_stride, weight);
     LLMS_LAUNCH_CHECK();
 }
 

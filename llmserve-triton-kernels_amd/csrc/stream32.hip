@@ -199,12 +199,14 @@ __global__ __launch_bounds__(S32_THREADS) void gated_add_kernel(float* __restric
 // One workgroup a row.  x_src is [N, S, hidden] (stream stride `hidden`) or, with src_broadcast, [N, hidden] read as
 // S equal copies; x_dst (may be x_src itself: every thread reads all of a column's streams before it writes them) takes
 // the new streams when `store`.  `y` null: nothing is added and the streams pass as they are.  `read` null: the plain
-// sum of the streams.  `rows`: only these rows are worked out (out[r] from row rows[r]).  Dynamic LDS: hidden floats.
+// sum of the streams.  `rows`: only these rows are worked out (out[r] from row rows[r]).  `center` 0: the mean is not
+// taken off (an RMS norm: u / sqrt(mean(u^2) + eps) * w).  Dynamic LDS: hidden floats.
 template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void streams_norm_kernel(
     T* __restrict__ out, float* x_dst, const float* x_src, int src_broadcast, const float* __restrict__ y,
     const float* __restrict__ mix, const float* __restrict__ wout, const float* __restrict__ read,
-    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store) {
+    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store,
+    int center) {
     extern __shared__ float u_row[];
     __shared__ float red[16];
     __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
@@ -247,7 +249,7 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_kernel(
         u_row[c] = u;
         total += u;
     }
-    const float mean = block_sum(total, red) / (float)hidden;
+    const float mean = center ? block_sum(total, red) / (float)hidden : 0.f;
     float dev2 = 0.f;
     for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
         const float d = u_row[c] - mean;
@@ -265,7 +267,8 @@ template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
     T* __restrict__ out, float* x_dst, const float* x_src, int src_broadcast, const float* __restrict__ y,
     const float* __restrict__ mix, const float* __restrict__ wout, const float* __restrict__ read,
-    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store) {
+    const float* __restrict__ weight, const int* __restrict__ rows, int streams, int hidden, float eps, int store,
+    int center) {
     extern __shared__ float u_row[];
     __shared__ float red[16];
     __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
@@ -332,7 +335,7 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
             total += (u.x + u.y) + (u.z + u.w);
         }
     }
-    const float mean = block_sum(total, red) / (float)hidden;
+    const float mean = center ? block_sum(total, red) / (float)hidden : 0.f;
     float dev2 = 0.f;
     for (int c4 = threadIdx.x; c4 < n4; c4 += S32_THREADS) {
         const float4 u = *reinterpret_cast<const float4*>(u_row + 4 * c4);
@@ -352,7 +355,31 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
     }
 }
 
+// x <- cap * tanh(x / cap), in place on 32-bit numbers (logits)
+__global__ void softcap_kernel(float* __restrict__ x, size_t total, float cap) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+// out = sa * a + sb * b (out may be a or b: a thread reads both before it writes)
+__global__ void weighted_sum_kernel(float* out, const float* a, const float* b, float sa, float sb, size_t total) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) out[i] = fmaf(sa, a[i], sb * b[i]);
+}
+
 extern "C" {
+
+int llms_weighted_sum(float* out, const float* a, const float* b, float sa, float sb, size_t total, hipStream_t stream) {
+    LLMS_REQUIRE(total > 0, "weighted_sum: a positive size");
+    weighted_sum_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(out, a, b, sa, sb, total);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_softcap(float* x, size_t total, float cap, hipStream_t stream) {
+    LLMS_REQUIRE(total > 0 && cap > 0.f, "softcap: a positive size and a positive cap");
+    softcap_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(x, total, cap);
+    LLMS_LAUNCH_CHECK();
+}
 
 int llms_embed_scale(int dtype, float* out, const void* table, const int* ids, int n, int hidden, int vocab, float scale,
                      hipStream_t stream) {
@@ -432,7 +459,7 @@ int llms_gated_add_norm(int dtype, void* out, float* x, const float* z, int z_st
 
 int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, int src_broadcast, const float* y,
                       const float* mix, const float* wout, const float* read, const float* weight, const int* rows,
-                      int n_out, int streams, int hidden, float eps, int store, hipStream_t stream) {
+                      int n_out, int streams, int hidden, float eps, int store, int center, hipStream_t stream) {
     LLMS_REQUIRE(n_out > 0 && hidden > 0, "streams_norm: sizes must be positive");
     LLMS_REQUIRE(streams >= 1 && streams <= STREAMS_MAX, "streams_norm: 1 to 8 streams");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "streams_norm: dtype must be 0 (float32) or 1 (bfloat16)");
@@ -446,7 +473,7 @@ int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, in
         if (lds > 32 * 1024)                                                                                                \
             LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)KERNEL<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)); \
         KERNEL<T><<<n_out, S32_THREADS, lds, stream>>>((T*)out, x_dst, x_src, src_broadcast, y, mix, wout, read, weight, rows, \
-                                                       streams, hidden, eps, store);                                        \
+                                                       streams, hidden, eps, store, center);                                \
     } while (0)
     if (vec && dtype == 0) STREAMS_GO(streams_norm_vec_kernel, float);
     else if (vec) STREAMS_GO(streams_norm_vec_kernel, bf16);

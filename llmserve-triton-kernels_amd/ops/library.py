@@ -752,6 +752,17 @@ def embed_scale(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale
     return out
 
 
+def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap) in place; x float32, contiguous."""
+    dev = _dev(x)
+    _f32(x, "x")
+    if not cap > 0:
+        raise ValueError("the cap must be positive")
+    if x.numel():
+        _check(load("stream32").llms_softcap(_ptr(x), ctypes.c_size_t(x.numel()), c_float(cap), _stream(dev)), "softcap")
+    return x
+
+
 def rmsnorm32(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float = 0.0,
               rows: torch.Tensor | None = None) -> torch.Tensor:
     """out[r] = x[s] / sqrt(mean(x[s]^2) + eps) * (offset + weight), s = rows[r] or r, all in 32-bit and rounded
@@ -941,6 +952,59 @@ def conv_state(state: torch.Tensor, proj: torch.Tensor, state_slots: torch.Tenso
         "conv_state")
 
 
+def _check_dist_bias_and_gate(dist_bias, gate, heads: int, dv: int, n: int) -> None:
+    if dist_bias is not None and (dist_bias.dtype != torch.float32 or dist_bias.dim() != 2 or dist_bias.shape[0] != heads
+                                  or dist_bias.shape[1] < 1 or not dist_bias.is_contiguous()):
+        raise ValueError(f"dist_bias must be a contiguous float32 [{heads}, R + 1] tensor")
+    if gate is not None and (gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != n
+                             or gate.shape[1] < heads * dv):
+        raise ValueError(f"gate must be float32 [{n}, >= {heads * dv}] with unit inner stride")
+
+
+def norm_store(q_out: torch.Tensor, proj: torch.Tensor, *, q_heads: int, k_heads: int, dk: int, v_heads: int, dv: int,
+               q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None, eps: float = 0.0,
+               temp_coef: float = 0.0, temp_every: int = 0, positions: torch.Tensor | None = None,
+               slots: torch.Tensor | None = None, k_pool: torch.Tensor | None = None, v_pool: torch.Tensor | None = None,
+               block_size: int = 0) -> torch.Tensor:
+    """proj float32 [N, >= q_heads*dk + k_heads*dk + v_heads*dv] (q, k, v side by side; unit inner stride): every
+    head of q and of k is divided by its root mean square (eps inside the root) and multiplied by `q_norm` / `k_norm`
+    (float32 [dk], shared by the heads; None: the head passes as it is); q is multiplied by
+    1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) at position p (temp_every 0: no factor); rounded once: queries
+    to q_out [N, q_heads*dk], keys and values to the tokens' cache slots (`slots`; None: nothing is stored)."""
+    dev = _dev(q_out, proj, q_norm, k_norm, positions, slots, k_pool, v_pool)
+    n = proj.shape[0]
+    channels = (q_heads + k_heads) * dk + v_heads * dv
+    if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] < channels:
+        raise ValueError(f"proj must be float32 [N, >= {channels}] with unit inner stride")
+    _rows(q_out, "q_out", q_heads * dk)
+    if q_out.shape[0] != n:
+        raise ValueError("q_out and proj differ in rows")
+    for t, name in ((q_norm, "q_norm"), (k_norm, "k_norm")):
+        if t is not None:
+            _f32(t, name, dk)
+    if temp_every < 0:
+        raise ValueError("temp_every must not be negative")
+    if temp_every > 0:
+        _i32(positions, "positions", n)
+    if slots is not None:
+        _i32(slots, "slots", n)
+        pages = k_pool.shape[0]
+        if tuple(k_pool.shape) != (pages, k_heads, block_size, dk) or not k_pool.is_contiguous():
+            raise ValueError(f"k_pool shape {tuple(k_pool.shape)} is not [pages,{k_heads},{block_size},{dk}]")
+        if tuple(v_pool.shape) != (pages, v_heads, dv, block_size) or not v_pool.is_contiguous():
+            raise ValueError(f"v_pool shape {tuple(v_pool.shape)} is not [pages,{v_heads},{dv},{block_size}]")
+        if k_pool.dtype != q_out.dtype or v_pool.dtype != q_out.dtype:
+            raise ValueError("pools and q_out differ in dtype")
+    if n == 0:
+        return q_out
+    _check(load("attention_composed").llms_norm_store(
+        c_int(_code(q_out)), _ptr(q_out), c_int(q_out.stride(0)), _ptr(proj), c_int(proj.stride(0)), _ptr(q_norm),
+        _ptr(k_norm), c_float(eps), c_float(temp_coef), c_int(temp_every), _ptr(positions), _ptr(slots), _ptr(k_pool),
+        _ptr(v_pool), c_int(n), c_int(q_heads), c_int(k_heads), c_int(dk), c_int(v_heads), c_int(dv), c_int(block_size),
+        _stream(dev)), "norm_store")
+    return q_out
+
+
 ATTEND_COMPOSED_LDS = 160 * 1024
 
 
@@ -957,7 +1021,8 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
                     keep_first: int = 0, chunk: int = 0, slopes: torch.Tensor | None = None,
                     talk: torch.Tensor | None = None, lam: float = 0.0, head_norm: bool = False, eps: float = 0.0,
                     out_scale: float = 1.0, table_rows: torch.Tensor | None = None,
-                    context_lens: torch.Tensor | None = None) -> torch.Tensor:
+                    context_lens: torch.Tensor | None = None, dist_bias: torch.Tensor | None = None,
+                    gate: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of N new tokens over the paged cache, one workgroup per token (all its heads), float32 or bfloat16
     storage, 32-bit arithmetic.  q [N, heads*maps*dk] (head by head, a head's maps side by side); k_pool
     [pages, kv_heads*maps, block, dk]; v_pool [pages, kv_heads, dv, block]; out [N, heads*dv].  A query at
@@ -965,8 +1030,12 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
     0).  `slopes` float32 [heads]: slope_h * (i - j) is taken off the scores.  `talk` float32 [heads, heads]: the
     heads' normalised weights are mixed, w_h = sum_g talk[h, g] w_g (maps = 1).  maps = 2: a_1 - lam * a_2.
     `head_norm`: each head's result is divided by its root mean square (eps inside the root) and multiplied by
-    out_scale.  `context_lens` [B]: rows of a request of length 0 are padding and give zeros."""
-    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions, slopes, talk, table_rows, context_lens)
+    out_scale.  `context_lens` [B]: rows of a request of length 0 are padding and give zeros.  `dist_bias` float32
+    [heads, R + 1]: dist_bias[h, min(i - j, R)] is added to the scores.  `gate` float32 [N, >= heads*dv] (unit inner
+    stride): the result is multiplied by sigmoid(gate)."""
+    dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions, slopes, talk, table_rows, context_lens,
+               dist_bias, gate)
+    _check_dist_bias_and_gate(dist_bias, gate, heads, dv, q.shape[0])
     n = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < heads * maps * dk:
         raise ValueError("q must be [N, >= heads*maps*dk] with unit inner stride")
@@ -1003,7 +1072,9 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
         _ptr(block_tables), _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(token_seq), _ptr(positions),
         _ptr(context_lens), c_int(n), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dk), c_int(dv),
         c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
-        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _stream(dev)),
+        c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _ptr(dist_bias),
+        c_int(dist_bias.shape[1] - 1 if dist_bias is not None else 0), _ptr(gate),
+        c_int(gate.stride(0) if gate is not None else 0), _stream(dev)),
         "attend_composed")
     return out
 
@@ -1130,11 +1201,11 @@ STREAMS_MAX = 8
 def streams_norm(out: torch.Tensor | None, x: torch.Tensor, weight: torch.Tensor | None, eps: float, *,
                  source: torch.Tensor | None = None, y: torch.Tensor | None = None, mix: torch.Tensor | None = None,
                  write: torch.Tensor | None = None, read: torch.Tensor | None = None,
-                 rows: torch.Tensor | None = None) -> torch.Tensor | None:
+                 rows: torch.Tensor | None = None, center: bool = True) -> torch.Tensor | None:
     """A residual stream of S copies x [N, S, hidden] (float32), in one kernel:
     with `y` [N, hidden] the streams become new_t = sum_s mix[s, t] x_s + write[t] y, all at once (stored into x
     unless `rows` picks rows); u = sum_t read[t] new_t (`read` None: the plain sum); out = layer norm of u with
-    `weight`, no bias, rounded once to out's dtype.  `source` [N, hidden]: the streams are read as S copies of it
+    `weight`, no bias, rounded once to out's dtype (`center` False: the mean is not taken off, an RMS norm).  `source` [N, hidden]: the streams are read as S copies of it
     (and stored into x).  `rows`: out[r] is worked out from row rows[r], nothing is stored.  `out` None: only the
     streams are brought up to date."""
     dev = _dev(out, x, weight, source, y, mix, write, read, rows)
@@ -1173,7 +1244,8 @@ def streams_norm(out: torch.Tensor | None, x: torch.Tensor, weight: torch.Tensor
     _check(load("stream32").llms_streams_norm(
         c_int(_code(out) if out is not None else 0), _ptr(out), _ptr(x), _ptr(src), c_int(source is not None), _ptr(y),
         _ptr(mix), _ptr(write), _ptr(read), _ptr(weight), _ptr(rows), c_int(n_out), c_int(s), c_int(hidden), c_float(eps),
-        c_int(1 if store and (y is not None or source is not None) else 0), _stream(dev)), "streams_norm")
+        c_int(1 if store and (y is not None or source is not None) else 0), c_int(1 if center else 0), _stream(dev)),
+        "streams_norm")
     return out
 
 
@@ -1346,6 +1418,7 @@ GROUPED_TILE = 64  # rows of a tile of the multiply-add kernel
 GROUPED_TILE_MFMA = 128  # and of the matrix-core kernel
 PAIRED_BLOCK = 32  # units per block of a paired weight: 32 rows of the first projection, then 32 of the second
 _EPILOGUES = {"plain": 0, "paired": 1, "gated": 2}
+_GATED_UNITS = {"clamped": 0, "silu": 1}
 GROUPED_KERNEL = os.environ.get("LLMSERVE_GROUPED_GEMM", "")  # "fma": keep the matrix-core kernel out
 
 
@@ -1370,13 +1443,15 @@ def _grouped_on_matrix_cores(x: torch.Tensor, w: torch.Tensor, x_ld: int, x_gs: 
 
 def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epilogue: str = "plain",
                     segments: "tuple[torch.Tensor, torch.Tensor] | None" = None, gate: torch.Tensor | None = None,
-                    gate_column: int = 0, limit: float = 0.0, units: int = 0, k_parts: int = 1) -> torch.Tensor:
+                    gate_column: int = 0, limit: float = 0.0, units: int = 0, k_parts: int = 1,
+                    unit: str = "clamped") -> torch.Tensor:
     """w [G, N, K].  Without `segments` every row meets every group: x [M, G, K] and out [M, G, N'] (views whose
     last axis has unit stride; the strides of the other two are free), out[m, g] = x[m, g] w[g]^T.  With `segments`
     = (seg [G + 1], tile_start [2, G + 1]) on the device (what `moe_sort` returns), x [M, K] and out [M, N'] hold rows
     sorted by group, rows seg[g] .. seg[g + 1] belonging to group g.
     Epilogues: "plain" (N' = N); "paired" (N' = `units`: w is `stack_paired(a, b)`,
-    out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1)); "gated" (out times
+    out = min(a, limit) sigmoid(1.702 min(a, limit)) (clamp(b, +-limit) + 1), or with `unit` "silu"
+    out = a sigmoid(a) b); "gated" (out times
     sigmoid(gate[m, gate_column + g N + n]), gate float32 [M, columns]).
     bfloat16 operands with K and the strides of x in multiples of 8 go to the matrix cores, all else to the 32-bit
     multiply-add kernel.  `k_parts` > 1 (as `grouped_k_parts` allows): out is float32 [k_parts, M, N] and holds partial
@@ -1392,6 +1467,8 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
     g, n, k = w.shape
     if epilogue not in _EPILOGUES:
         raise ValueError(f"epilogue {epilogue!r}")
+    if unit not in _GATED_UNITS:
+        raise ValueError(f"unit {unit!r}; choose from {sorted(_GATED_UNITS)}")
     if epilogue == "paired" and (n % (2 * PAIRED_BLOCK) or not 0 < units <= n // 2):
         raise ValueError(f"a paired weight of {n} rows does not hold {units} units")
     n_out = units if epilogue == "paired" else n
@@ -1436,7 +1513,7 @@ def grouped_product(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, *, epil
         return out
     common = (_ptr(out), c_long(out_ld), c_long(out_gs), _ptr(x), c_long(x_ld), c_long(x_gs), _ptr(w), c_int(m), c_int(n),
               c_int(k), c_int(g), _ptr(seg_ptr), _ptr(tiles_ptr), c_int(max_tiles), _ptr(z), c_long(z_ld), c_long(z_gs),
-              c_float(limit), c_int(units), _stream(dev))
+              c_float(limit), c_int(_GATED_UNITS[unit]), c_int(units), _stream(dev))
     lib = load("grouped_gemm")
     if mfma:
         _check(lib.llms_grouped_mfma(c_int(_code(out)), c_int(_EPILOGUES[epilogue]), *common[:-1], c_int(k_parts),
@@ -1463,10 +1540,13 @@ MOE_MAX_TOP = 16
 
 
 def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_router: torch.Tensor, *,
-               renormalize: bool = False) -> None:
-    """Per row of h [N, hidden]: scores sigmoid(W_router h) in 32-bit, the `top` largest in descending order (the
-    lower expert wins a tie) into chosen int32 [N, top], their scores (over their sum with `renormalize`) into
-    weight float32 [N, top]."""
+               renormalize: bool = False, scores: str = "sigmoid", groups: int = 1, keep: int = 1,
+               renorm_eps: float = 0.0) -> None:
+    """Per row of h [N, hidden]: scores sigmoid(W_router h), or with `scores` "softmax" the softmax over all experts,
+    in 32-bit; the `top` largest in descending order (the lower expert wins a tie) into chosen int32 [N, top], their
+    scores (over their sum + `renorm_eps` with `renormalize`) into weight float32 [N, top].  `groups` > 1: the experts
+    form that many equal groups of neighbours, a group's score is its largest, and only experts of the `keep` best
+    groups can be chosen."""
     dev = _dev(chosen, weight, h, w_router)
     _rows(h, "h")
     _rows(w_router, "w_router", h.shape[1])
@@ -1478,11 +1558,16 @@ def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_ro
         raise ValueError("h and w_router differ in dtype")
     if not 1 <= top <= min(MOE_MAX_TOP, experts):
         raise ValueError(f"1 to {MOE_MAX_TOP} choices among {experts} experts, got {top}")
+    if scores not in ("sigmoid", "softmax"):
+        raise ValueError(f"scores {scores!r}; choose 'sigmoid' or 'softmax'")
+    if groups < 1 or experts % groups or not 1 <= keep <= groups or (groups > 1 and top > keep * (experts // groups)):
+        raise ValueError(f"{groups} groups of which {keep} are kept do not fit {experts} experts and {top} choices")
     if n == 0:
         return
     _check(load("moe").llms_moe_router(
         c_int(_code(h)), _ptr(chosen), _ptr(weight), _ptr(h), _ptr(w_router), c_int(n), c_int(h.shape[1]), c_int(experts),
-        c_int(top), c_int(1 if renormalize else 0), _stream(dev)), "moe_router")
+        c_int(top), c_int(1 if renormalize else 0), c_int(1 if scores == "softmax" else 0), c_int(groups), c_int(keep),
+        c_float(renorm_eps), _stream(dev)), "moe_router")
 
 
 def moe_sort(chosen: torch.Tensor, experts: int):
@@ -1502,9 +1587,10 @@ def moe_sort(chosen: torch.Tensor, experts: int):
     return rank, seg, tiles
 
 
-def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor,
-                rank: torch.Tensor, seg: torch.Tensor) -> None:
-    """xs[seg[chosen[p]] + rank[p]] = weight[p] * h[p // top] (rounded to xs's dtype); place[p] = that row."""
+def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor,
+                weight: torch.Tensor | None, rank: torch.Tensor, seg: torch.Tensor) -> None:
+    """xs[seg[chosen[p]] + rank[p]] = weight[p] * h[p // top] (rounded to xs's dtype; `weight` None: the row as it
+    is); place[p] = that row."""
     dev = _dev(xs, place, h, chosen, weight, rank, seg)
     _rows(h, "h")
     pairs = chosen.numel()
@@ -1516,17 +1602,19 @@ def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: 
     _i32(chosen, "chosen", pairs)
     _i32(rank, "rank", pairs)
     _i32(seg, "seg")
-    _f32(weight, "weight", pairs)
+    if weight is not None:
+        _f32(weight, "weight", pairs)
     if pairs == 0:
         return
     _check(load("moe").llms_moe_scatter(c_int(_code(h)), _ptr(xs), _ptr(place), _ptr(h), _ptr(chosen), _ptr(weight), _ptr(rank),
                                         _ptr(seg), c_int(pairs), c_int(h.shape[1]), c_int(top), _stream(dev)), "moe_scatter")
 
 
-def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor) -> torch.Tensor:
-    """y[n] = sum_k rows[place[n, k]] in the order of k; y float32 [N, hidden], rows float32 [pairs, hidden] or
-    [parts, pairs, hidden] (partial sums of each row, added in the order of the parts)."""
-    dev = _dev(y, rows, place)
+def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
+    """y[n] = sum_k rows[place[n, k]] in the order of k (times weight[n, k] where `weight`, float32 [N, top], is
+    given); y float32 [N, hidden], rows float32 [pairs, hidden] or [parts, pairs, hidden] (partial sums of each row,
+    added in the order of the parts)."""
+    dev = _dev(y, rows, place, weight)
     n, hidden = y.shape
     _f32(y, "y")
     _f32(rows, "rows")
@@ -1536,8 +1624,128 @@ def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor) -> tor
     top = pairs // max(n, 1)
     if rows.shape[-1] != hidden or top * n != pairs:
         raise ValueError("rows has top rows of y's width per row of y")
+    if weight is not None:
+        _f32(weight, "weight", pairs)
     if n == 0:
         return y
     _check(load("moe").llms_moe_combine(_ptr(y), _ptr(rows), _ptr(place), c_int(n), c_int(hidden), c_int(top), c_int(parts),
-                                        c_long(pairs * hidden), _stream(dev)), "moe_combine")
+                                        c_long(pairs * hidden), _ptr(weight), _stream(dev)), "moe_combine")
     return y
+
+
+# ------------------------------------------------------------------------------ linear attention with a decay per head
+
+DECAY_MAX_KEY = 256  # numbers of a key that `decay_scan` takes
+_ACTIVATIONS = {None: 0, "none": 0, "silu": 1, "sigmoid": 2}
+
+
+def _decay_proj(proj: torch.Tensor, col_q: int, col_k: int, col_v: int, heads: int, dk: int, dv: int) -> None:
+    if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1:
+        raise ValueError("proj must be a float32 [N, columns] tensor with unit inner stride")
+    for col, width, name in ((col_q, heads * dk, "q"), (col_k, heads * dk, "k"), (col_v, heads * dv, "v")):
+        if col < 0 or col + width > proj.shape[1]:
+            raise ValueError(f"the columns of {name} ({col} .. {col + width}) lie outside proj's {proj.shape[1]}")
+
+
+def decay_prepare(proj: torch.Tensor, *, col_q: int, col_k: int, col_v: int, heads: int, dk: int, dv: int,
+                  activation: str | None = None, freq: torch.Tensor | None = None, rot_dims: int = 0,
+                  positions: torch.Tensor | None = None, key_scale: float = 1.0) -> torch.Tensor:
+    """In place on proj float32 [N, columns] (q, k and v of `heads` heads from the given columns on): `activation`
+    ("silu" or None) on q, k and v; with `freq` float32 [rot_dims / 2], dimension i < rot_dims / 2 of every head of q and
+    k is turned together with dimension i + rot_dims / 2 by the angle positions[n] * freq[i]; k times `key_scale`."""
+    dev = _dev(proj, freq, positions)
+    _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
+    if activation not in (None, "none", "silu"):
+        raise ValueError(f"activation {activation!r}; choose 'silu' or None")
+    if rot_dims:
+        if rot_dims % 2 or not 0 < rot_dims <= dk:
+            raise ValueError(f"{rot_dims} turned dimensions of {dk}")
+        _f32(freq, "freq", rot_dims // 2)
+        _i32(positions, "positions", proj.shape[0])
+    if proj.shape[0] == 0:
+        return proj
+    _check(load("decay_attention").llms_decay_prepare(
+        _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v), _ptr(positions if rot_dims else None),
+        _ptr(freq if rot_dims else None), c_int(rot_dims), c_int(proj.shape[0]), c_int(heads), c_int(dk), c_int(dv),
+        c_int(_ACTIVATIONS[activation]), c_float(key_scale), _stream(dev)), "decay_prepare")
+    return proj
+
+
+def _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv) -> int:
+    if state.dtype != torch.float32 or not state.is_contiguous() or tuple(state.shape[1:]) != (heads, dk, dv):
+        raise ValueError(f"state must be a contiguous float32 [slots, {heads}, {dk}, {dv}] tensor")
+    _i32(cu_seqlens, "cu_seqlens")
+    b = cu_seqlens.numel() - 1
+    _i32(state_slots, "state_slots", b)
+    _i32(context_lens, "context_lens", b)
+    _f32(decay, "decay", heads)
+    return b
+
+
+def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+               cu_seqlens: torch.Tensor, context_lens: torch.Tensor, decay: torch.Tensor, *, col_q: int, col_k: int,
+               col_v: int, heads: int, dk: int, dv: int) -> torch.Tensor:
+    """The recurrence S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t over the new tokens of every request, token by
+    token: request b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of proj (float32; q, k, v from the given columns on),
+    starts from state[state_slots[b]] (float32 [slots, heads, dk, dv]; from zero when its portion starts at position 0,
+    which context_lens[b], its length after the step, tells) and leaves its last state there.  out float32 [N, heads*dv].
+    A request of length 0 is padding: its rows give zeros and no state is touched."""
+    dev = _dev(out, proj, state, state_slots, cu_seqlens, context_lens, decay)
+    _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
+    if out.dtype != torch.float32 or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (proj.shape[0], heads * dv):
+        raise ValueError(f"out must be float32 [{proj.shape[0]}, {heads * dv}] with unit inner stride")
+    if dk > DECAY_MAX_KEY:
+        raise ValueError(f"keys of up to {DECAY_MAX_KEY} numbers, got {dk}")
+    b = _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv)
+    if b <= 0 or proj.shape[0] == 0:
+        return out
+    _check(load("decay_attention").llms_decay_scan(
+        _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
+        _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), c_int(b), c_int(heads), c_int(dk),
+        c_int(dv), _stream(dev)), "decay_scan")
+    return out
+
+
+def decay_finish(out: torch.Tensor, o: torch.Tensor, *, heads: int, dv: int, eps: float, weight: torch.Tensor | None = None,
+                 gate: torch.Tensor | None = None, gate_activation: str | None = None) -> torch.Tensor:
+    """out[n] = norm(o[n]) * activation(gate[n]), rounded once to out's dtype.  o float32 [N, heads*dv].  `weight` None:
+    every head is divided by its own root mean square (eps inside the root); `weight` float32 [heads*dv]: all heads
+    together are RMS-normed and multiplied by it.  `gate` float32 [N, >= heads*dv] (unit inner stride) with
+    `gate_activation` "sigmoid" or "silu"."""
+    dev = _dev(out, o, weight, gate)
+    width = heads * dv
+    if o.dtype != torch.float32 or o.dim() != 2 or o.stride(1) != 1 or o.shape[1] != width:
+        raise ValueError(f"o must be float32 [N, {width}] with unit inner stride")
+    _rows(out, "out", width)
+    n = o.shape[0]
+    if out.shape[0] != n:
+        raise ValueError("out and o differ in rows")
+    if weight is not None:
+        _f32(weight, "weight", width)
+    if gate_activation not in (None, "none", "silu", "sigmoid"):
+        raise ValueError(f"gate_activation {gate_activation!r}")
+    act = _ACTIVATIONS[gate_activation]
+    if act:
+        if gate is None or gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != n \
+                or gate.shape[1] < width:
+            raise ValueError(f"gate must be float32 [{n}, >= {width}] with unit inner stride")
+    if width * 4 > 128 * 1024:
+        raise ValueError("heads times value size up to 32,768")
+    if n == 0:
+        return out
+    _check(load("decay_attention").llms_decay_finish(
+        c_int(_code(out)), _ptr(out), c_int(out.stride(0)), _ptr(o), c_int(o.stride(0)), _ptr(gate if act else None),
+        c_int(gate.stride(0) if act else 0), _ptr(weight), c_int(n), c_int(heads), c_int(dv), c_int(1 if weight is not None else 0),
+        c_int(act), c_float(eps), _stream(dev)), "decay_finish")
+    return out
+
+
+def weighted_sum(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, scale_a: float, scale_b: float) -> torch.Tensor:
+    """out = scale_a * a + scale_b * b, element by element in 32-bit (out may be a or b)."""
+    dev = _dev(out, a, b)
+    for t, name in ((out, "out"), (a, "a"), (b, "b")):
+        _f32(t, name, out.numel())
+    if out.numel():
+        _check(load("stream32").llms_weighted_sum(_ptr(out), _ptr(a), _ptr(b), c_float(scale_a), c_float(scale_b),
+                                                  ctypes.c_size_t(out.numel()), _stream(dev)), "weighted_sum")
+    return out

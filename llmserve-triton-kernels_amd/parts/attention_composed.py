@@ -16,8 +16,17 @@ Parameters (a `PartSpec` of kind "composed_attention"):
                         o = a_1 - lambda a_2 with lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + `diff`
   head_norm_eps         each head's result is divided by its root mean square (eps inside the root), no weight,
                         and multiplied by `head_norm_scale` (None: no such norm)
+  bias                  q, k and v have biases (tensors "<name>.b"), added in the projection
+  qk_norm_eps           every head of q and of k is RMS-normed over its dk numbers with a weight of size dk that all
+                        heads share (tensors "q.norm", "k.norm"; eps inside the root); None: no such norm
+  query_temperature     {coef, every}: q at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1)
+  distance_table        {rows: B, farthest: D}: a learned bias per head and distance, tensor "rel" [B, H], added to the
+                        scaled score: rel[bucket(i - j), h] with bucket(n) = n for n < B/2 and
+                        min(B - 1, B/2 + floor(ln(n / (B/2)) / ln(D / (B/2)) (B - B/2))) beyond
+  output_gate           the heads' results are multiplied by sigmoid(W_g h) (tensor "g") before the output projection
   result                "float32": the output projection's result stays unrounded (for a 32-bit residual stream)
-  names                 local tensor names (defaults: q, k, v, o, q.conv, k.conv, v.conv, talk, lq1, lk1, lq2, lk2)
+  names                 local tensor names (defaults: q, k, v, o, q.conv, k.conv, v.conv, talk, lq1, lk1, lq2, lk2,
+                        q.b, k.b, v.b, q.norm, k.norm, rel, g)
 
 Scores, softmax, the mixing of heads, the difference of the maps and the head norm are computed in 32-bit; the
 convolution is computed in 32-bit from the unrounded projection and rounded once.  Keys are cached as [pages,
@@ -37,7 +46,34 @@ from .registry import Mixer, register_mixer
 from .spec import PagedCacheSpec, ParamInfo, StateCacheSpec
 
 _DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "q_conv": "q.conv", "k_conv": "k.conv", "v_conv": "v.conv",
-                  "talk": "talk", "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2"}
+                  "talk": "talk", "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2", "q_bias": "q.b", "k_bias": "k.b",
+                  "v_bias": "v.b", "q_norm": "q.norm", "k_norm": "k.norm", "rel": "rel", "g": "g"}
+
+
+def distance_bucket(n: int, rows: int, farthest: int) -> int:
+    """Row of a distance table of `rows` rows for the distance n >= 0: a row per distance below rows / 2, then rows
+    whose spans grow geometrically up to `farthest`; everything beyond shares the last row."""
+    half = rows // 2
+    if n < half:
+        return n
+    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(farthest / half) * (rows - half))))
+
+
+def bias_by_distance(table: torch.Tensor, farthest: int) -> torch.Tensor:
+    """table [rows, H] -> float32 [H, R + 1] with the bias of every distance 0 .. R, R being the first distance from
+    which the last row holds for good: what the attention kernels index by min(i - j, R)."""
+    rows = table.shape[0]
+    reach = max(int(farthest), rows // 2)
+    while reach > 0 and distance_bucket(reach - 1, rows, farthest) == rows - 1:
+        reach -= 1
+    index = torch.tensor([distance_bucket(n, rows, farthest) for n in range(reach + 1)], dtype=torch.long,
+                         device=table.device)
+    return table.float()[index].t().contiguous()
+
+
+def _fill_rel(shape, generator, device, options):
+    """A distance table: moderate biases."""
+    return 0.5 * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
 
 
 def _fill_taps(shape, generator, device, options):
@@ -78,6 +114,21 @@ class ComposedAttention(Mixer):
         self.result_dtype = torch.float32 if spec.get("result", "model") == "float32" else None
         self.names = dict(_DEFAULT_NAMES, **(spec.get("names") or {}))
         self.maps = 2 if self.differential else 1
+        self.bias = bool(spec.get("bias", False))
+        self.qk_norm_eps = spec.get("qk_norm_eps")
+        temp = spec.get("query_temperature") or {}
+        self.temp_coef, self.temp_every = float(temp.get("coef", 0.0)), int(temp.get("every", 0))
+        table = spec.get("distance_table")
+        self.rel_rows = int(table["rows"]) if table else 0
+        self.rel_farthest = int(table["farthest"]) if table else 0
+        self.output_gate = bool(spec.get("output_gate", False))
+        if table and (self.rel_rows < 2 or self.rel_farthest <= self.rel_rows // 2):
+            raise ValueError("a distance table has at least 2 rows and reaches beyond the distances that have a row each")
+        if (self.qk_norm_eps is not None or self.temp_every) and self.taps > 0:
+            raise ValueError("normed or position-scaled queries do not go together with a convolution")
+        if self.temp_every < 0:
+            raise ValueError("query_temperature.every must be positive")
+        self.dist_bias = self.q_norm = self.k_norm = self.in_bias = None
         if self.num_heads % self.num_kv_heads:
             raise ValueError("num_heads must be a multiple of num_kv_heads")
         for name in ("window", "chunk"):
@@ -122,13 +173,33 @@ class ComposedAttention(Mixer):
         if self.differential:
             for key in ("lq1", "lk1", "lq2", "lk2"):
                 infos[n[key]] = ParamInfo((self.head_dim,), "around_zero")
+        if self.bias:
+            for key, channels in (("q_bias", self.cq), ("k_bias", self.ck), ("v_bias", self.cv)):
+                infos[n[key]] = ParamInfo((channels,), "around_zero")
+        if self.qk_norm_eps is not None:
+            infos[n["q_norm"]] = ParamInfo((self.head_dim,), "norm")
+            infos[n["k_norm"]] = ParamInfo((self.head_dim,), "norm")
+        if self.rel_rows:
+            infos[n["rel"]] = ParamInfo((self.rel_rows, self.num_heads), _fill_rel)
+        if self.output_gate:
+            infos[n["g"]] = ParamInfo((self.num_heads * self.value_dim, h))
         return infos
 
     def load(self, tensors):
         n = self.names
         dev = tensors[n["q"]].device
-        self.qkv_weight = torch.cat([tensors[n[x]] for x in "qkv"], dim=0).contiguous()
+        pieces = [tensors[n[x]] for x in "qkv"] + ([tensors[n["g"]]] if self.output_gate else [])
+        self.qkv_weight = torch.cat(pieces, dim=0).contiguous()  # (the gate's rows lie behind those of q, k and v)
         self.o_weight = tensors[n["o"]].contiguous()
+        if self.bias:
+            biases = [tensors[n[x + "_bias"]] for x in "qkv"]
+            if self.output_gate:
+                biases.append(torch.zeros(self.num_heads * self.value_dim, dtype=biases[0].dtype, device=dev))
+            self.in_bias = torch.cat(biases).contiguous()
+        if self.qk_norm_eps is not None:
+            self.q_norm, self.k_norm = tensors[n["q_norm"]].float().contiguous(), tensors[n["k_norm"]].float().contiguous()
+        if self.rel_rows:
+            self.dist_bias = bias_by_distance(tensors[n["rel"]], self.rel_farthest)
         if self.taps > 0:
             self.taps_w = torch.cat([tensors[n[x + "_conv"]].float() for x in "qkv"], dim=0).contiguous()
         if self.talking:
@@ -145,8 +216,8 @@ class ComposedAttention(Mixer):
     @property
     def input_weight(self):
         """The stacked q, k, v projection: an arrangement may fold it into a product of its own (32-bit result) and
-        hand the result back as `projected`."""
-        return self.qkv_weight
+        hand the result back as `projected`.  (None where the projection has biases, which such a product lacks.)"""
+        return None if self.bias else self.qkv_weight
 
     @input_weight.setter
     def input_weight(self, weight):
@@ -157,8 +228,20 @@ class ComposedAttention(Mixer):
         view = batch.groups[paged.group_id]
         heads, kv, dk, dv = self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim
         # q, k and v side by side, unrounded
-        proj = projected if projected is not None else linear(x, self.qkv_weight, out_dtype=torch.float32)
+        proj = projected if projected is not None else linear(x, self.qkv_weight, self.in_bias, out_dtype=torch.float32)
         q = torch.empty((proj.shape[0], self.cq), dtype=x.dtype, device=x.device)
+        gate = proj[:, self.cq + self.ck + self.cv:] if self.output_gate else None
+        if self.qk_norm_eps is not None or self.temp_every:
+            ops.norm_store(q, proj, q_heads=heads * self.maps, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,
+                           q_norm=self.q_norm, k_norm=self.k_norm, eps=float(self.qk_norm_eps or 0.0),
+                           temp_coef=self.temp_coef, temp_every=self.temp_every, positions=batch.positions,
+                           slots=view.slots if paged.store else None, k_pool=paged.k_pool, v_pool=paged.v_pool,
+                           block_size=paged.block_size)
+            out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
+            self.attend(out, q, paged, view, batch, gate)
+            return linear(out, self.o_weight, out_dtype=self.result_dtype)
+        if self.output_gate:
+            proj = proj[:, : self.cq + self.ck + self.cv]
         conv, taps = self.taps > 1, self.taps > 0  # (one tap is a factor per channel and needs no state)
         single = conv and batch.max_count == 1 and batch.num_seqs == proj.shape[0]  # every request brings one token
         ops.conv_store(q, proj, cq=self.cq, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,
@@ -171,10 +254,10 @@ class ComposedAttention(Mixer):
         if conv and not single:
             ops.conv_state(state.state, proj, batch.state_slots, batch.cu_seqlens, batch.context_lens)
         out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
-        self.attend(out, q, paged, view, batch)
+        self.attend(out, q, paged, view, batch, gate)
         return linear(out, self.o_weight, out_dtype=self.result_dtype)
 
-    def attend(self, out, q, paged, view, batch):
+    def attend(self, out, q, paged, view, batch, gate=None):
         """out[n] = this attention of token n's heads over its request's pages: on the matrix cores where the
         sizes allow (bfloat16; requests that bring one token in one launch, portions of prompts in another), else
         by the kernel that takes any size and dtype."""
@@ -183,10 +266,10 @@ class ComposedAttention(Mixer):
                       keep_first=self.keep_first, chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk,
                       lam=self.lam, head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
                       out_scale=self.head_norm_scale, table_rows=batch.state_slots)
-        if not ops.attend_composed_mfma_supported(q.dtype, self.num_heads, self.num_kv_heads, self.head_dim,
-                                                  self.value_dim, paged.block_size, self.talking):
+        if self.dist_bias is not None or gate is not None or not ops.attend_composed_mfma_supported(
+                q.dtype, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, paged.block_size, self.talking):
             ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
-                                context_lens=batch.context_lens, **common)
+                                context_lens=batch.context_lens, dist_bias=self.dist_bias, gate=gate, **common)
             return
         args = (out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         n_dec = batch.num_decode

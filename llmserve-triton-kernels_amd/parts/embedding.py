@@ -50,8 +50,8 @@ class TokenEmbedding(Part):
 
 @HEADS.register("lm_head")
 class LMHead(Part):
-    """Parameters: vocab, hidden, tied.  A tied head has no tensor of its own: the model
-    hands it the embedding table."""
+    """Parameters: vocab, hidden, tied, tensor, softcap.  A tied head has no tensor of its own: the model
+    hands it the embedding table.  `softcap` c: the logits become c tanh(logits / c), in 32-bit."""
     graph_safe = True
     accepts_deferred_norm = True  # (when every row's logits are wanted the model hands over the final norm's input)
 
@@ -61,7 +61,11 @@ class LMHead(Part):
         self.hidden = int(spec["hidden"])
         self.tied = bool(spec.get("tied", False))
         self.tensor = spec.get("tensor", "weight")  # the matrix's local name
+        self.softcap = None if spec.get("softcap") is None else float(spec["softcap"])
         self.weight: torch.Tensor | None = None
+
+    def libraries(self, dtype_name):
+        return ("stream32",) if self.softcap is not None else ()
 
     def param_infos(self):
         return {} if self.tied else {self.tensor: ParamInfo((self.vocab, self.hidden))}
@@ -70,6 +74,10 @@ class LMHead(Part):
         self.weight = tensors["weight" if self.tied else self.tensor].contiguous()
 
     def forward(self, h) -> torch.Tensor:
+        logits = self._logits(h)
+        return logits if self.softcap is None else ops.softcap(logits, self.softcap)
+
+    def _logits(self, h) -> torch.Tensor:
         if isinstance(h, DeferredNorm):
             rows, norm = h.residual, h.fused()
             if norm is not None and rows.shape[0] <= ops.GEMM_DECODE_NORM_ROWS and decode_product(rows, self.weight):

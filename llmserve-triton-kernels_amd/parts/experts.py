@@ -2,11 +2,16 @@
 
 Parameters (a `PartSpec` of kind "experts"): hidden, intermediate (of one expert), experts, top, limit,
 renormalize (default False: the weights are the chosen scores as they are), names (local names: "router", and the
-pattern of an expert's matrices, default "e{e}.gate", "e{e}.up", "e{e}.down").
+pattern of an expert's matrices, default "e{e}.gate", "e{e}.up", "e{e}.down"), and, with defaults that leave them
+out: scores ("sigmoid" or "softmax" over all experts), groups and keep (the experts form `groups` equal groups of
+neighbours, a group's score is its largest, only experts of the `keep` best groups can be chosen), renorm_eps (added
+to the sum that `renormalize` divides by), weight_on ("input": the weight multiplies the expert's input; "output":
+its result), unit ("clamped" or "silu").
 
-Router: z = W_router h in 32-bit, scores sigmoid(z), the `top` largest chosen.  The weight multiplies the expert's
-*input*: y = sum over chosen e of expert_e(w_e h).  Expert: a = min(W_gate x, limit), b = clamp(W_up x, -limit,
-limit), W_down (a sigmoid(1.702 a) (b + 1)).  No biases.
+Router: z = W_router h in 32-bit, scores sigmoid(z) or softmax(z), the `top` largest chosen.  With weight_on
+"input" y = sum over chosen e of expert_e(w_e h), with "output" y = sum of w_e expert_e(h).  Expert, unit "clamped":
+a = min(W_gate x, limit), b = clamp(W_up x, -limit, limit), W_down (a sigmoid(1.702 a) (b + 1)); unit "silu":
+W_down (a sigmoid(a) b) with a = W_gate x, b = W_up x.  No biases.
 
 One step: route, sort the (token, choice) pairs by expert on the device (stably, so a pair's place does not depend
 on what else is in the batch beyond which rows share its tile), scatter the weighted inputs into that order, two
@@ -36,8 +41,21 @@ class Experts(FeedForward):
         self.intermediate = int(spec["intermediate"])
         self.experts = int(spec["experts"])
         self.top = int(spec["top"])
-        self.limit = float(spec["limit"])
+        self.unit = spec.get("unit", "clamped")
+        self.limit = float(spec["limit"]) if self.unit == "clamped" else 0.0
         self.renormalize = bool(spec.get("renormalize", False))
+        self.renorm_eps = float(spec.get("renorm_eps", 0.0))
+        self.scores = spec.get("scores", "sigmoid")
+        self.groups = int(spec.get("groups") or 1)
+        self.keep = int(spec.get("keep") or self.groups)
+        self.weight_on = spec.get("weight_on", "input")
+        if self.unit not in ("clamped", "silu") or self.scores not in ("sigmoid", "softmax") or \
+                self.weight_on not in ("input", "output"):
+            raise ValueError(f"unit={self.unit!r}, scores={self.scores!r}, weight_on={self.weight_on!r}")
+        if self.experts % self.groups or not 1 <= self.keep <= self.groups or \
+                (self.groups > 1 and self.top > self.keep * (self.experts // self.groups)):
+            raise ValueError(f"{self.groups} groups of which {self.keep} are kept do not fit {self.experts} experts "
+                             f"of which {self.top} are chosen")
         self.names = dict(_DEFAULT_NAMES, **(spec.get("names") or {}))
         if not 1 <= self.top <= min(self.experts, ops.MOE_MAX_TOP):
             raise ValueError(f"top={self.top} of {self.experts} experts (at most {ops.MOE_MAX_TOP})")
@@ -69,17 +87,20 @@ class Experts(FeedForward):
         pairs = rows * self.top
         chosen = torch.empty((rows, self.top), dtype=torch.int32, device=dev)
         weight = torch.empty((rows, self.top), dtype=torch.float32, device=dev)
-        ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize)
+        ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize, scores=self.scores,
+                       groups=self.groups, keep=self.keep, renorm_eps=self.renorm_eps)
+        on_input = self.weight_on == "input"
         rank, seg, tiles = ops.moe_sort(chosen, self.experts)
         sorted_in = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
         place = torch.empty(pairs, dtype=torch.int32, device=dev)
-        ops.moe_scatter(sorted_in, place, x, chosen, weight, rank, seg)
+        ops.moe_scatter(sorted_in, place, x, chosen, weight if on_input else None, rank, seg)
         act = torch.empty((pairs, self.intermediate), dtype=x.dtype, device=dev)
         ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit,
-                            units=self.intermediate)
+                            units=self.intermediate, unit=self.unit)
         # (few rows: the last product's K is shared out, and the sum over a token's choices adds the shares up as well)
         parts = ops.grouped_k_parts(act, self.w_down, ops.compute_units(dev))
         shape = (pairs, self.hidden) if parts == 1 else (parts, pairs, self.hidden)
         results = torch.empty(shape, dtype=torch.float32, device=dev)
         ops.grouped_product(results, act, self.w_down, segments=(seg, tiles), k_parts=parts)
-        return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place)
+        return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place,
+                               None if on_input else weight)

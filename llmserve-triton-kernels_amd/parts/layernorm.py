@@ -20,6 +20,7 @@ from .spec import ParamInfo
 class LayerNorm32(Norm):
     graph_safe = True
     closes_streams = True  # `read_streams`, `add_norm` and `norm_rows` take an `OpenStreams` in the place of delta
+    center = True  # the mean is taken off
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -57,7 +58,8 @@ class LayerNorm32(Norm):
         x = self._streams(x)
         out = torch.empty((x.shape[0], self.hidden), dtype=self.ctx.dtype, device=x.device)
         read = None if connection is None else connection.read
-        return ops.streams_norm(out, x, self.weight, self.eps, source=source, read=read, **self._open(delta))
+        return ops.streams_norm(out, x, self.weight, self.eps, source=source, read=read, center=self.center,
+                                **self._open(delta))
 
     def forward(self, x):
         return self.read_streams(x, None)
@@ -68,7 +70,15 @@ class LayerNorm32(Norm):
     def norm_rows(self, x, delta, rows):
         x = self._streams(x)
         out = torch.empty((rows.numel(), self.hidden), dtype=self.ctx.dtype, device=x.device)
-        return ops.streams_norm(out, x, self.weight, self.eps, rows=rows, **self._open(delta))
+        return ops.streams_norm(out, x, self.weight, self.eps, rows=rows, center=self.center, **self._open(delta))
+
+
+@register_norm("rmsnorm_streams")
+class RMSNormStreams(LayerNorm32):
+    """The same over the same streams without taking the mean off: u / sqrt(mean(u^2) + eps) * w, all in 32-bit,
+    rounded once.  Parameters as above."""
+
+    center = False
 
 
 @register_norm("none")

@@ -11,8 +11,8 @@ from __future__ import annotations
 
 import torch
 
-from . import (attention, attention_composed, attention_latent, block, connection, embedding, experts, gate,  # noqa: F401
-               layernorm, rmsnorm, rope, swiglu)  # (register the built-in parts)
+from . import (attention, attention_composed, attention_latent, block, connection, decay_attention, embedding,  # noqa: F401
+               experts, gate, layernorm, rmsnorm, rope, side_by_side, swiglu)  # (register the built-in parts)
 from .registry import BLOCKS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
 from .spec import ModelSpec, ParamInfo
 
