@@ -42,11 +42,10 @@ def distance_bucket(n: int, rows: int, farthest: int) -> int:
 def distance_bias(t: int, table: torch.Tensor, farthest: int) -> torch.Tensor:
     """[H, T, T]: table[bucket(i - j), h] for j <= i (0 elsewhere)."""
     rows, heads = table.shape
-    out = torch.zeros((heads, t, t), dtype=table.dtype)
-    for i in range(t):
-        for j in range(i + 1):
-            out[:, i, j] = table[distance_bucket(i - j, rows, farthest)]
-    return out
+    row_of = torch.tensor([distance_bucket(n, rows, farthest) for n in range(t)], dtype=torch.long)
+    distance = torch.arange(t)[:, None] - torch.arange(t)[None, :]
+    bias = table[row_of[distance.clamp(min=0)]]  # [T, T, H]
+    return (bias * (distance >= 0)[:, :, None]).permute(2, 0, 1)
 
 
 def query_temperature(t: int, coef: float, every: int, dtype) -> torch.Tensor:
@@ -181,7 +180,10 @@ def forward(config: dict, tensors: dict, tokens, dtype=torch.float64, layers_out
     eps = float(config["norm"]["eps"])
     x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * float(config["embedding"]["scale"])
     for i, entry in enumerate(config["layers"]):
-        p = f"l{entry.get('weights_of', i)}."
+        owner = i
+        while config["layers"][owner].get("weights_of") is not None:  # (a layer may name one that names another)
+            owner = int(config["layers"][owner]["weights_of"])
+        p = f"l{owner}."
         mix = {k[len(p) + 4:]: v for k, v in w.items() if k.startswith(p + "mix.")}
         h = rms_norm(x, w[p + "norm1"], eps)
         if entry["type"] == "parallel":
@@ -198,3 +200,13 @@ def forward(config: dict, tensors: dict, tokens, dtype=torch.float64, layers_out
     logits = rms_norm(x, w["final.norm"], eps) @ w["head"].T
     cap = config.get("logit_softcap")
     return logits if cap is None else float(cap) * torch.tanh(logits / float(cap))
+
+
+def greedy(config: dict, tensors: dict, prompt, n_new: int) -> list[int]:
+    """The `n_new` tokens of largest logit, one after the other (the lowest index wins a tie)."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        token = int(forward(config, tensors, ids)[-1].argmax())
+        out.append(token)
+        ids.append(token)
+    return out
