@@ -26,9 +26,10 @@ first token, inter-token latency percentiles and the number of preemptions besid
 `--pages-fraction` shrinks the cache pool below what the whole workload needs, so that
 requests wait and are preempted.
 
-    python bench.py --workload designs [--design dibepel|milozen] [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
+    python bench.py --workload designs [--design dibepel|milozen|felavik] [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
 
-puts the Dibepel design (or, with `--design milozen`, the Milozen design: latent attention, experts, two streams)
+puts the Dibepel design (or, with `--design milozen`, the Milozen design: latent attention, experts, two streams; with
+`--design felavik`, the Felavik design: linear attention with a decay per head, gated softmax attention, experts in groups)
 beside the Llama decoder at equal layer sizes (width, heads, key/value heads, head size,
 feed-forward, vocabulary, layers; random weights): prefill tokens a second for one prompt of 2,048 tokens in one
 step, and decoded tokens a second at the given batch sizes behind `--context` tokens, both through the step
@@ -236,6 +237,38 @@ def milozen_config(size: dict, layers: int, window: int = 1024, experts: int = 8
             "norm": {"eps": 1e-5}, "streams": streams, "layers": entries}
 
 
+def felavik_config(size: dict, layers: int, experts: int = 8, top: int = 2) -> dict:
+    """Linear attention with as many heads of the head size as the Llama shape (keys and values of the head size); every
+    fourth layer from the second instead has the gated softmax attention of the Llama shape's heads and key/value heads
+    beside a retention of half as many heads, the last such layer on the tensors of the first; every layer chooses `top`
+    of `experts` experts (in 4 groups of which 2 are kept) that together are as wide as the dense feed-forward."""
+    dim, heads = size["dim"], size["heads"]
+
+    def decays(n):
+        return [1.0 - 2.0 ** (-5.0 - 5.0 * k / max(n - 1, 1)) for k in range(n)]
+
+    mlp = {"kind": "moe", "expert": {"ff": size["ff"] // top},
+           "router": {"experts": experts, "top": top, "groups": {"count": 4, "keep": 2}}}
+    entries, first = [], None
+    for i in range(layers):
+        if i % 4 == 1:
+            entry = {"type": "parallel", "mlp": mlp, "mixer": {
+                "left": {"heads": heads, "kv_heads": size["kv_heads"], "dim": dim, "vdim": dim, "scale": dim ** -0.5,
+                         "bias_max": 1024, "bias_rows": 32, "q_temp": {"coef": 0.1, "every": 1024}},
+                "right": {"heads": heads // 2, "dim": dim, "vdim": dim, "decay": decays(heads // 2),
+                          "rot": {"base": 10000.0, "dims": dim}},
+                "left_scale": 1.0, "right_scale": 1.0}}
+            if first is None:
+                first = i
+            else:
+                entry["weights_of"] = first
+        else:
+            entry = {"type": "lightning", "mlp": mlp, "mixer": {"heads": heads, "dim": dim, "vdim": dim, "decay": decays(heads)}}
+        entries.append(entry)
+    return {"architecture": "Felavik", "vocab": size["vocab"], "width": size["width"], "embedding": {"scale": 1.0},
+            "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": entries}
+
+
 def llama_config(size: dict, layers: int, positions: int) -> dict:
     return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=size["vocab"], hidden_size=size["width"],
                 intermediate_size=size["ff"], num_hidden_layers=layers, num_attention_heads=size["heads"],
@@ -310,7 +343,7 @@ def designs(args) -> int:
 
     table = {}
     design = args.design
-    make = {"dibepel": dibepel_config, "milozen": milozen_config}[design]
+    make = {"dibepel": dibepel_config, "milozen": milozen_config, "felavik": felavik_config}[design]
     for name in [s for s in args.sizes.split(",") if s]:
         size = DESIGN_SIZES[name]
         layers = args.layers or 6
@@ -452,7 +485,7 @@ def main() -> int:
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
                          "decode products alone, each over copies of its weight that do not fit the caches")
     ap.add_argument("--workload", choices=["steps", "serve", "designs"], default="steps")
-    ap.add_argument("--design", choices=["dibepel", "milozen"], default="dibepel", help="designs: which design stands beside Llama")
+    ap.add_argument("--design", choices=["dibepel", "milozen", "felavik"], default="dibepel", help="designs: which design stands beside Llama")
     ap.add_argument("--sizes", default="1b,7b", help="designs: layer sizes to compare at")
     ap.add_argument("--batches", default="8,32", help="designs: decode batch sizes")
     ap.add_argument("--requests", type=int, default=64)

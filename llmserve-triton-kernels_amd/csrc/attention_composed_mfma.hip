@@ -50,6 +50,9 @@ struct MfmaArgs {
     const int* context_lens;
     const float* slopes;
     const float* talk;
+    const float* dist_bias;  // [heads, dist_reach + 1]: a bias per head and distance, the last entry for everything beyond; or null
+    const float* gate;       // 32-bit products [N, gate_stride]: the result is multiplied by their sigmoid; or null
+    int dist_reach, gate_stride;
     int out_stride, q_stride, max_blocks;
     int seq_begin, n_seqs, blocks_per_seq;
     int heads, kv_heads, grp, dk, dv, block_size;
@@ -143,7 +146,8 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     // this wave's units and columns
     bool valid[MAXU], mine[MAXU];
     int u_kvh[MAXU], u_h[MAXU], u_tl[MAXU], u_pos[MAXU], u_chunk_lo[MAXU];
-    float u_slope[MAXU];
+    float u_slope[MAXU], u_far[MAXU];
+    const float* u_bias[MAXU];  // the column's head's row of the distance table
     int u_pmin[MAXU], u_pmax[MAXU];
     s16x4 qf[MAXU][MAPS][MAXTK];
 #pragma unroll
@@ -156,6 +160,8 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         u_kvh[uu] = kvh, u_h[uu] = h, u_tl[uu] = tl, u_pos[uu] = pos_lo + tl;
         u_chunk_lo[uu] = a.chunk > 0 ? u_pos[uu] / a.chunk * a.chunk : 0;
         u_slope[uu] = (a.slopes && valid[uu]) ? a.slopes[h] * LOG2E : 0.f;
+        u_bias[uu] = a.dist_bias ? a.dist_bias + (size_t)(valid[uu] ? h : 0) * (a.dist_reach + 1) : nullptr;
+        u_far[uu] = a.dist_bias ? u_bias[uu][a.dist_reach] * LOG2E : 0.f;
         // the unit's first and last position (the same for all its lanes): a tile that all of them see whole
         // needs no comparisons
         u_pmin[uu] = pos_lo + sub * a.tpw;
@@ -243,6 +249,22 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
                     const bool vis = valid[uu] && key <= pos && key >= u_chunk_lo[uu] &&
                                      (a.window <= 0 || pos - key < a.window || key < a.keep_first);
                     sc[tt][r] = vis ? acc[r] * scale2 - u_slope[uu] * (dist0 - (float)r) : -INFINITY;
+                }
+            }
+            if (a.dist_bias) {  // the table's entry of every key's distance; a tile that lies beyond the table's reach for all has one
+                const int d0 = pos - j0 - 4 * q4;
+                if (__all(d0 - 3 >= a.dist_reach)) {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sc[tt][r] += u_far[uu];
+                } else {
+                    float bias[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {  // (a key that is not seen holds -inf already; its entry is read from a place that exists)
+                        const int d = d0 - r;
+                        bias[r] = u_bias[uu][d < 0 ? 0 : (d < a.dist_reach ? d : a.dist_reach)];
+                    }
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sc[tt][r] = fmaf(bias[r], LOG2E, sc[tt][r]);
                 }
             }
         }
@@ -566,10 +588,16 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
             continue;
         }
         bf16* orow = a.out + (size_t)(row0 + t0 + u_tl[uu]) * a.out_stride + (size_t)u_h[uu] * dv + 4 * q4;
+        const float* grow = a.gate ? a.gate + (size_t)(row0 + t0 + u_tl[uu]) * a.gate_stride + (size_t)u_h[uu] * dv + 4 * q4 : nullptr;
 #pragma unroll
         for (int t = 0; t < MAXTV; ++t)
             if (t < dvt) {
-                const f32x4 o = acc_o[uu][0][t] * norm;
+                f32x4 o = acc_o[uu][0][t] * norm;
+                if (grow) {
+                    const f32x4 z = *reinterpret_cast<const f32x4*>(grow + 16 * t);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) o[r] /= 1.f + expf(-z[r]);
+                }
                 *reinterpret_cast<s16x4*>(orow + 16 * t) = pack4(o[0], o[1], o[2], o[3]);
             }
     }
@@ -637,7 +665,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
                               int heads, int kv_heads, int maps, int dk, int dv, int block_size, int window,
                               int keep_first, int chunk, float scale, const float* slopes, const float* talk, float lambda,
                               int head_norm, float eps, float out_scale, int shares, float* ws_stats, float* ws_o, int ws_rows,
-                              hipStream_t stream) {
+                              const float* dist_bias, int dist_reach, const float* gate, int gate_stride, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && kv_heads > 0, "attend_composed_mfma: sizes must be positive");
     LLMS_REQUIRE(heads % kv_heads == 0 && heads / kv_heads <= 16, "attend_composed_mfma: up to 16 query heads per key/value head");
     LLMS_REQUIRE(maps == 1 || maps == 2, "attend_composed_mfma: one or two score maps");
@@ -651,6 +679,9 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.out = (bf16*)out, a.q = (const bf16*)q, a.k_pool = (const bf16*)k_pool, a.v_pool = (const bf16*)v_pool;
     a.block_tables = block_tables, a.table_rows = table_rows, a.cu_seqlens = cu_seqlens, a.context_lens = context_lens;
     a.slopes = slopes, a.talk = talk;
+    LLMS_REQUIRE(!dist_bias || dist_reach >= 0, "attend_composed_mfma: a distance table has at least one entry per head");
+    LLMS_REQUIRE(!gate || (!talk && gate_stride % 4 == 0), "attend_composed_mfma: gate rows are 16-byte aligned, and no gate where heads are mixed");
+    a.dist_bias = dist_bias, a.dist_reach = dist_reach, a.gate = gate, a.gate_stride = gate_stride;
     a.out_stride = out_stride, a.q_stride = q_stride, a.max_blocks = max_blocks, a.seq_begin = seq_begin, a.n_seqs = n_seqs;
     a.heads = heads, a.kv_heads = kv_heads, a.grp = heads / kv_heads, a.dk = dk, a.dv = dv, a.block_size = block_size;
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;

@@ -123,6 +123,181 @@ __global__ __launch_bounds__(DA_THREADS) void decay_scan_kernel(
     }
 }
 
+// ---- portions of many tokens: runs of DA_CHUNK tokens on the 32-bit matrix instruction ------------------------------
+//
+// A run is DA_CHUNK (64) neighbouring new tokens of one request, counted from the start of its portion (any cut gives the
+// same recurrence).  Its place in the workspace [runs, heads, dk, dv] is cu_seqlens[b] / 64 + b + j (run j of request b):
+// the runs of different requests never meet, and N / 64 + requests places hold them all.
+// All three kernels form products of 32 x 32 tiles with v_mfma_f32_32x32x2_f32 (true 32-bit operands and sums):
+// lane l brings A[l % 32][l / 32] and B[l / 32][l % 32] of a step of 2, and holds the 16 numbers
+// C[8 (i / 4) + 4 (l / 32) + i % 4][l % 32], i = 0 .. 15.  Operands lie in LDS, rows padded by one number.
+#define DA_CHUNK 64
+#define DA_SLAB 64  // columns of v (and of the state) that a workgroup takes
+
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+// powers[n] = decay^n, n = 0 .. DA_CHUNK, by repeated multiplication (any decay, also 0 and negative ones)
+__device__ __forceinline__ void da_powers(float* powers, float d) {
+    if (threadIdx.x == 0) {
+        double p = 1.0;
+        for (int n = 0; n <= DA_CHUNK; ++n) powers[n] = (float)p, p *= (double)d;
+    }
+}
+
+__device__ __forceinline__ int da_run_place(int row0, int b, int j) { return row0 / DA_CHUNK + b + j; }
+
+// grid: (runs of the longest portion, heads, requests * slabs).  ws[run][h] = sum_t decay^(n - 1 - t) k_t v_t^T over the
+// run's n tokens.
+template <int DKP>
+__global__ __launch_bounds__(DA_THREADS) void decay_chunk_sums_kernel(
+    float* __restrict__ ws, const float* __restrict__ proj, int stride, int col_k, int col_v,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens, const float* __restrict__ decay, int heads,
+    int dk, int dv, int slabs) {
+    constexpr int LD = DKP + 1, LV = DA_SLAB + 1;
+    __shared__ float ks[DA_CHUNK * LD];
+    __shared__ float vs[DA_CHUNK * LV];
+    __shared__ float powers[DA_CHUNK + 1];
+    const int b = blockIdx.z / slabs, c0 = (blockIdx.z % slabs) * DA_SLAB, h = blockIdx.y, j = blockIdx.x;
+    const int row0 = cu_seqlens[b], count = cu_seqlens[b + 1] - row0;
+    if (context_lens[b] <= 0 || j * DA_CHUNK >= count) return;
+    const int n = min(DA_CHUNK, count - j * DA_CHUNK);
+    da_powers(powers, decay[h]);
+    __syncthreads();
+    const float* rows = proj + (size_t)(row0 + j * DA_CHUNK) * stride;
+    for (int e = threadIdx.x; e < DA_CHUNK * DKP; e += DA_THREADS) {
+        const int t = e / DKP, i = e % DKP;
+        ks[t * LD + i] = (t < n && i < dk) ? rows[(size_t)t * stride + col_k + h * dk + i] * powers[n - 1 - t] : 0.f;
+    }
+    for (int e = threadIdx.x; e < DA_CHUNK * DA_SLAB; e += DA_THREADS) {
+        const int t = e / DA_SLAB, c = e % DA_SLAB;
+        vs[t * LV + c] = (t < n && c0 + c < dv) ? rows[(size_t)t * stride + col_v + h * dv + c0 + c] : 0.f;
+    }
+    __syncthreads();
+    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, lo = lane % 32, hi = lane / 32;
+    float* dst = ws + ((size_t)da_run_place(row0, b, j) * heads + h) * dk * dv;
+    for (int tile = wave; tile < (DKP / 32) * (DA_SLAB / 32); tile += DA_THREADS / LLMS_WAVE) {
+        const int ir = tile / (DA_SLAB / 32) * 32, tc = tile % (DA_SLAB / 32) * 32;
+        f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 8
+        for (int t = 0; t < DA_CHUNK; t += 2)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ks[(t + hi) * LD + ir + lo], vs[(t + hi) * LV + tc + lo], acc, 0, 0, 0);
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+            const int i = ir + 8 * (x / 4) + 4 * hi + x % 4, c = c0 + tc + lo;
+            if (i < dk && c < dv) dst[(size_t)i * dv + c] = acc[x];
+        }
+    }
+}
+
+// grid: (ceil(dk dv / 256), heads, requests).  Turns the runs' sums into the state before each run, in place, and stores
+// the request's last state.
+__global__ __launch_bounds__(DA_THREADS) void decay_chunk_scan_kernel(
+    float* __restrict__ ws, float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ context_lens, const float* __restrict__ decay, int heads, int dk, int dv) {
+    const int b = blockIdx.z, h = blockIdx.y, e = blockIdx.x * DA_THREADS + threadIdx.x;
+    const int row0 = cu_seqlens[b], count = cu_seqlens[b + 1] - row0, length = context_lens[b];
+    if (length <= 0 || count <= 0 || e >= dk * dv) return;
+    const float d = decay[h];
+    double full = 1.0, rest = 1.0;
+    const int runs = (count + DA_CHUNK - 1) / DA_CHUNK, last = count - (runs - 1) * DA_CHUNK;
+    for (int n = 0; n < DA_CHUNK; ++n) {
+        full *= (double)d;
+        if (n < last) rest *= (double)d;
+    }
+    float* st = state + ((size_t)state_slots[b] * heads + h) * dk * dv + e;
+    float s = length > count ? *st : 0.f;  // (a portion from position 0 starts from zero)
+    float* at = ws + ((size_t)da_run_place(row0, b, 0) * heads + h) * dk * dv + e;
+    const size_t step = (size_t)heads * dk * dv;
+    float sum = *at;
+    for (int j = 0; j < runs; ++j) {
+        const float next = j + 1 < runs ? at[step] : 0.f;  // (asked for before this run's is overwritten and used)
+        *at = s;
+        s = fmaf(j + 1 < runs ? (float)full : (float)rest, s, sum);
+        sum = next, at += step;
+    }
+    *st = s;
+}
+
+// grid: (runs of the longest portion, heads, requests * slabs).  o_t = decay^(t + 1) S^T q_t + sum_(s <= t) (q_t . k_s)
+// decay^(t - s) v_s over the run's tokens, S being the state before the run (ws[run][h]).
+template <int DKP>
+__global__ __launch_bounds__(DA_THREADS) void decay_chunk_out_kernel(
+    float* __restrict__ out, int out_stride, const float* __restrict__ ws, const float* __restrict__ proj, int stride, int col_q,
+    int col_k, int col_v, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+    const float* __restrict__ decay, int heads, int dk, int dv, int slabs) {
+    constexpr int LD = DKP + 1, LV = DA_SLAB + 1, LP = DA_CHUNK + 1;
+    constexpr int KS = DA_CHUNK * LD > DKP * LV ? DA_CHUNK * LD : DKP * LV;  // the keys, and after them the state's columns
+    extern __shared__ float lds[];
+    float* qs = lds;                    // [64][LD]
+    float* ks = qs + DA_CHUNK * LD;     // [64][LD], later ss [DKP][LV]
+    float* ps = ks + KS;                // [64][LP]
+    float* vs = ps + DA_CHUNK * LP;     // [64][LV]
+    float* powers = vs + DA_CHUNK * LV; // [65]
+    const int b = blockIdx.z / slabs, c0 = (blockIdx.z % slabs) * DA_SLAB, h = blockIdx.y, j = blockIdx.x;
+    const int row0 = cu_seqlens[b], count = cu_seqlens[b + 1] - row0;
+    if (j * DA_CHUNK >= count) return;
+    const int n = min(DA_CHUNK, count - j * DA_CHUNK);
+    if (context_lens[b] <= 0) {  // padding: no request, no state; its rows leave zeros
+        for (int e = threadIdx.x; e < n * DA_SLAB; e += DA_THREADS)
+            if (c0 + e % DA_SLAB < dv) out[(size_t)(row0 + j * DA_CHUNK + e / DA_SLAB) * out_stride + h * dv + c0 + e % DA_SLAB] = 0.f;
+        return;
+    }
+    da_powers(powers, decay[h]);
+    const float* rows = proj + (size_t)(row0 + j * DA_CHUNK) * stride;
+    for (int e = threadIdx.x; e < DA_CHUNK * DKP; e += DA_THREADS) {
+        const int t = e / DKP, i = e % DKP;
+        const bool there = t < n && i < dk;
+        qs[t * LD + i] = there ? rows[(size_t)t * stride + col_q + h * dk + i] : 0.f;
+        ks[t * LD + i] = there ? rows[(size_t)t * stride + col_k + h * dk + i] : 0.f;
+    }
+    for (int e = threadIdx.x; e < DA_CHUNK * DA_SLAB; e += DA_THREADS) {
+        const int t = e / DA_SLAB, c = e % DA_SLAB;
+        vs[t * LV + c] = (t < n && c0 + c < dv) ? rows[(size_t)t * stride + col_v + h * dv + c0 + c] : 0.f;
+    }
+    __syncthreads();
+    const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, lo = lane % 32, hi = lane / 32;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    {   // what the run's tokens see of each other: tiles (0,0), (1,0), (1,1) of q k^T, each weighted by the decay over the
+        // distance; tile (0,1) lies ahead of its queries
+        const int tr = wave == 0 ? 0 : 32, tc = wave == 2 ? 32 : 0;
+        f32x16 acc = zero;
+        if (wave < 3) {
+#pragma unroll 8
+            for (int i = 0; i < DKP; i += 2)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qs[(tr + lo) * LD + i + hi], ks[(tc + lo) * LD + i + hi], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+            const int t = (wave == 3 ? 0 : tr) + 8 * (x / 4) + 4 * hi + x % 4, s2 = (wave == 3 ? 32 : tc) + lo;
+            ps[t * LP + s2] = (wave < 3 && s2 <= t) ? acc[x] * powers[t - s2] : 0.f;
+        }
+    }
+    __syncthreads();  // (the keys are done with)
+    float* ss = ks;
+    const float* before = ws + ((size_t)da_run_place(row0, b, j) * heads + h) * dk * dv;
+    for (int e = threadIdx.x; e < DKP * DA_SLAB; e += DA_THREADS) {
+        const int i = e / DA_SLAB, c = e % DA_SLAB;
+        ss[i * LV + c] = (i < dk && c0 + c < dv) ? before[(size_t)i * dv + c0 + c] : 0.f;
+    }
+    __syncthreads();
+    const int tr = (wave % 2) * 32, tc = (wave / 2) * 32;
+    f32x16 acc = zero;
+#pragma unroll 8
+    for (int i = 0; i < DKP; i += 2)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qs[(tr + lo) * LD + i + hi], ss[(i + hi) * LV + tc + lo], acc, 0, 0, 0);
+#pragma unroll
+    for (int x = 0; x < 16; ++x) acc[x] *= powers[tr + 8 * (x / 4) + 4 * hi + x % 4 + 1];
+    const int keys = tr + 32;  // (the keys behind the tile's last query weigh nothing)
+#pragma unroll 8
+    for (int s2 = 0; s2 < keys; s2 += 2)
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(ps[(tr + lo) * LP + s2 + hi], vs[(s2 + hi) * LV + tc + lo], acc, 0, 0, 0);
+#pragma unroll
+    for (int x = 0; x < 16; ++x) {
+        const int t = tr + 8 * (x / 4) + 4 * hi + x % 4, c = c0 + tc + lo;
+        if (t < n && c < dv) out[(size_t)(row0 + j * DA_CHUNK + t) * out_stride + h * dv + c] = acc[x];
+    }
+}
+
 // grid: tokens.  Dynamic LDS: heads * dv floats.
 template <typename T>
 __global__ __launch_bounds__(DA_THREADS) void decay_finish_kernel(
@@ -195,6 +370,46 @@ int llms_decay_scan(float* out, int out_stride, const float* proj, int stride, i
     else if (dk <= 64) DA_GO(16);
     else if (dk <= 128) DA_GO(32);
     else DA_GO(64);
+#undef DA_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+// Floats of the workspace that `llms_decay_chunks` needs for n_tokens rows of n_seqs requests.
+long long llms_decay_chunks_workspace(int n_tokens, int n_seqs, int heads, int dk, int dv) {
+    return ((long long)n_tokens / DA_CHUNK + n_seqs + 1) * heads * dk * dv;
+}
+
+// The same recurrence as llms_decay_scan for portions of many tokens (`max_new`: the most one request brings).
+int llms_decay_chunks(float* out, int out_stride, const float* proj, int stride, int col_q, int col_k, int col_v, float* state,
+                      const int* state_slots, const int* cu_seqlens, const int* context_lens, const float* decay, float* ws,
+                      int n_seqs, int max_new, int heads, int dk, int dv, hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && dk > 0 && dv > 0, "decay_chunks: sizes must be positive");
+    LLMS_REQUIRE(dk <= 128, "decay_chunks: keys of up to 128 numbers");
+    LLMS_REQUIRE(ws, "decay_chunks: a workspace");
+    const int slabs = (dv + DA_SLAB - 1) / DA_SLAB, runs = (max_new + DA_CHUNK - 1) / DA_CHUNK;
+    LLMS_REQUIRE(heads <= 65535 && (long long)n_seqs * slabs <= 65535, "decay_chunks: up to 65,535 heads, and requests times slabs");
+    const dim3 grid(runs, heads, n_seqs * slabs);
+    const int dkp = (dk + 31) / 32 * 32;
+#define DA_GO(DKP)                                                                                                        \
+    do {                                                                                                                  \
+        decay_chunk_sums_kernel<DKP><<<grid, DA_THREADS, 0, stream>>>(ws, proj, stride, col_k, col_v, cu_seqlens,          \
+                                                                      context_lens, decay, heads, dk, dv, slabs);         \
+        decay_chunk_scan_kernel<<<dim3((dk * dv + DA_THREADS - 1) / DA_THREADS, heads, n_seqs), DA_THREADS, 0, stream>>>(   \
+            ws, state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv);                                      \
+        constexpr int ks = DA_CHUNK * (DKP + 1) > DKP * (DA_SLAB + 1) ? DA_CHUNK * (DKP + 1) : DKP * (DA_SLAB + 1);       \
+        const size_t lds = (size_t)(DA_CHUNK * (DKP + 1) + ks + DA_CHUNK * (DA_CHUNK + 1) + DA_CHUNK * (DA_SLAB + 1) +    \
+                                    DA_CHUNK + 1) * sizeof(float);                                                        \
+        if (lds > 48 * 1024)                                                                                              \
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)decay_chunk_out_kernel<DKP>,                                  \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                    \
+        decay_chunk_out_kernel<DKP><<<grid, DA_THREADS, lds, stream>>>(out, out_stride, ws, proj, stride, col_q, col_k,    \
+                                                                       col_v, cu_seqlens, context_lens, decay, heads, dk, \
+                                                                       dv, slabs);                                        \
+    } while (0)
+    if (dkp == 32) DA_GO(32);
+    else if (dkp == 64) DA_GO(64);
+    else if (dkp == 96) DA_GO(96);
+    else DA_GO(128);
 #undef DA_GO
     LLMS_LAUNCH_CHECK();
 }

@@ -1104,14 +1104,15 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
                          block_size: int, scale: float, maps: int = 1, window: int = 0, keep_first: int = 0,
                          chunk: int = 0, slopes: torch.Tensor | None = None, talk: torch.Tensor | None = None,
                          lam: float = 0.0, head_norm: bool = False, eps: float = 0.0, out_scale: float = 1.0,
-                         table_rows: torch.Tensor | None = None, shares: int = 1) -> torch.Tensor:
+                         table_rows: torch.Tensor | None = None, shares: int = 1, dist_bias: torch.Tensor | None = None,
+                         gate: torch.Tensor | None = None) -> torch.Tensor:
     """`attend_composed` on the matrix cores (bfloat16) for requests [seq_begin, seq_begin + n_seqs) of a step: request
     b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out, brings at most `max_new` tokens and is context_lens[b]
     long after the step (0: padding, left alone).  Same arguments and arithmetic otherwise; the weights are rounded
     to bfloat16 as the operand of the value product.  `shares` > 1 (where the heads' weights are mixed): the keys
     of every block of tokens are shared out to that many workgroups in two launches (maxima and sums; weights and
     values), their 32-bit parts added up by a third."""
-    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, slopes, talk, table_rows)
+    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, slopes, talk, table_rows, dist_bias, gate)
     if not attend_composed_mfma_supported(q.dtype, heads, kv_heads, dk, dv, block_size, talk is not None):
         raise ValueError("attend_composed_mfma does not take these sizes; see attend_composed_mfma_supported")
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < heads * maps * dk or q.stride(0) % 4 or q.data_ptr() % 8:
@@ -1143,6 +1144,13 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
         _f32(slopes, "slopes", heads)
     if talk is not None:
         _f32(talk, "talk", heads * heads)
+    if dist_bias is not None and (dist_bias.dtype != torch.float32 or dist_bias.dim() != 2 or dist_bias.shape[0] != heads
+                                  or dist_bias.shape[1] < 1 or not dist_bias.is_contiguous()):
+        raise ValueError("dist_bias must be a contiguous float32 [heads, reach + 1] tensor")
+    if gate is not None and (talk is not None or gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1
+                             or gate.shape[0] != q.shape[0] or gate.shape[1] < heads * dv or gate.stride(0) % 4
+                             or gate.data_ptr() % 16):
+        raise ValueError("gate must be float32 [N, >= heads*dv] with unit inner stride and 16-byte aligned rows (and no mixed heads)")
     if n_seqs == 0 or max_new <= 0 or q.shape[0] == 0:
         return out
     ws_stats = ws_o = None
@@ -1158,7 +1166,8 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
         c_int(n_seqs), c_int(max_new), c_int(heads), c_int(kv_heads), c_int(maps), c_int(dk), c_int(dv),
         c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
         c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), c_int(shares), _ptr(ws_stats),
-        _ptr(ws_o), c_int(q.shape[0]), _stream(dev)),
+        _ptr(ws_o), c_int(q.shape[0]), _ptr(dist_bias), c_int(dist_bias.shape[1] - 1 if dist_bias is not None else 0),
+        _ptr(gate), c_int(gate.stride(0) if gate is not None else 0), _stream(dev)),
         "attend_composed_mfma")
     return out
 
@@ -1703,6 +1712,36 @@ def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state
         _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
         _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), c_int(b), c_int(heads), c_int(dk),
         c_int(dv), _stream(dev)), "decay_scan")
+    return out
+
+
+DECAY_CHUNKS_MAX_KEY = 128  # numbers of a key that `decay_chunks` takes
+
+
+def decay_chunks(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                 cu_seqlens: torch.Tensor, context_lens: torch.Tensor, decay: torch.Tensor, max_new: int, *, col_q: int,
+                 col_k: int, col_v: int, heads: int, dk: int, dv: int) -> torch.Tensor:
+    """What `decay_scan` computes, for portions of many tokens (`max_new`: the most one request brings): runs of 64
+    tokens gather their own sums of k v^T, a scan over the runs gives the state before each and the request's last
+    state, and every run adds what its tokens see of each other to what they see of that state; all products on the
+    32-bit matrix instruction.  Same arguments, and the same result up to the order of the sums."""
+    dev = _dev(out, proj, state, state_slots, cu_seqlens, context_lens, decay)
+    _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
+    if out.dtype != torch.float32 or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (proj.shape[0], heads * dv):
+        raise ValueError(f"out must be float32 [{proj.shape[0]}, {heads * dv}] with unit inner stride")
+    if dk > DECAY_CHUNKS_MAX_KEY:
+        raise ValueError(f"keys of up to {DECAY_CHUNKS_MAX_KEY} numbers, got {dk}")
+    b = _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv)
+    if b <= 0 or proj.shape[0] == 0 or max_new <= 0:
+        return out
+    lib = load("decay_attention")
+    lib.llms_decay_chunks_workspace.restype = ctypes.c_longlong
+    floats = int(lib.llms_decay_chunks_workspace(c_int(proj.shape[0]), c_int(b), c_int(heads), c_int(dk), c_int(dv)))
+    ws = torch.empty(floats, dtype=torch.float32, device=dev)
+    _check(lib.llms_decay_chunks(
+        _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
+        _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), _ptr(ws), c_int(b), c_int(max_new),
+        c_int(heads), c_int(dk), c_int(dv), _stream(dev)), "decay_chunks")
     return out
 
 

@@ -37,6 +37,7 @@ _DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "norm": "nor
 @register_mixer("decay_attention")
 class DecayAttention(Mixer):
     graph_safe = True
+    SCAN_UP_TO = 16  # new tokens of the longest portion up to which the recurrence runs token by token
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -112,5 +113,10 @@ class DecayAttention(Mixer):
         return linear(out, self.o_weight, out_dtype=self.result_dtype)
 
     def recur(self, o, proj, state, batch, cols):
-        """o[n] = S^T q over the step's tokens, and the requests' states brought up to date."""
+        """o[n] = S^T q over the step's tokens, and the requests' states brought up to date: token by token where every
+        request brings few, in runs of 64 tokens on the matrix cores where one brings many."""
+        if batch.max_count > self.SCAN_UP_TO and self.head_dim <= ops.DECAY_CHUNKS_MAX_KEY:
+            ops.decay_chunks(o, proj, state, batch.state_slots, batch.cu_seqlens, batch.context_lens, self.decay,
+                             batch.max_count, **cols)
+            return
         ops.decay_scan(o, proj, state, batch.state_slots, batch.cu_seqlens, batch.context_lens, self.decay, **cols)
