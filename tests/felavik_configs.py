@@ -71,4 +71,15 @@ def _small_c():
     return config_of(layers, width=40, vocab=131, scale=0.8)
 
 
-SMALL, SMALL_B, SMALL_C = _small(), _small_b(), _small_c()
+def _small_d():
+    # sizes that the matrix cores take (multiples of 16), pages of 16 keys, a table that most keys lie beyond
+    layers = [lightning(heads=2, dim=16, vdim=48, decay=[0.7, 0.99]),
+              parallel(left={"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "bias_max": 24, "bias_rows": 12,
+                             "q_temp": {"coef": 0.4, "every": 16}},
+                       right={"heads": 2, "dim": 32, "vdim": 16, "decay": [0.9, 0.999], "rot": {"base": 1000.0, "dims": 16}}),
+              lightning(heads=1, dim=64, vdim=32, decay=[0.98], mlp=moe(4, 2, 32, 2, 1))]
+    layers.append(again(layers, 1))
+    return config_of(layers, width=64, vocab=173, scale=1.2)
+
+
+SMALL, SMALL_B, SMALL_C, SMALL_D = _small(), _small_b(), _small_c(), _small_d()

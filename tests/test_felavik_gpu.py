@@ -14,7 +14,7 @@ import torch
 
 import plain_felavik as pf
 import traces
-from felavik_configs import SMALL, SMALL_B, SMALL_C, config_of, lightning, moe, parallel
+from felavik_configs import SMALL, SMALL_B, SMALL_C, SMALL_D, config_of, lightning, moe, parallel
 
 pytestmark = pytest.mark.gpu
 
@@ -75,14 +75,20 @@ def test_activation_rotation_and_key_scale(heads, dk, dv, dims, act):
 SCAN_CASES = [(3, 12, 20), (2, 16, 8), (1, 72, 80), (2, 130, 70), (1, 32, 64), (5, 8, 200)]
 
 
+@pytest.mark.parametrize("kernel", ["scan", "chunks"])
 @pytest.mark.parametrize("heads,dk,dv", SCAN_CASES)
-def test_the_recurrence_in_portions_of_any_size_beside_each_other(heads, dk, dv):
+def test_the_recurrence_in_portions_of_any_size_beside_each_other(heads, dk, dv, kernel):
     """Three requests of unequal length advance in portions of changing size, down to one token, in one launch each
     step; between them sits a request of length 0 (padding).  Foreign state slots hold NaN; a slot that a finished
-    request gives back is used again by the next without being cleared by anyone but the kernel's own start."""
+    request gives back is used again by the next without being cleared by anyone but the kernel's own start.  Token by
+    token, and in runs of 64 tokens (portions of one run, of a run and one token, of several runs and a rest, and of
+    one token beside them)."""
     from llmserve.ops import library as ops
 
-    lengths = {"a": 61, "b": 9, "c": 33, "d": 20}
+    chunks = kernel == "chunks"
+    if chunks and dk > ops.DECAY_CHUNKS_MAX_KEY:
+        pytest.skip("keys wider than the kernel of runs takes")
+    lengths = {"a": 331, "b": 9, "c": 133, "d": 90} if chunks else {"a": 61, "b": 9, "c": 33, "d": 20}
     decay = [0.5 + 0.5 * (h + 1) / (heads + 1) for h in range(heads)]
     decay[-1] = 1.0 if heads > 1 else 0.97
     data = {r: (rnd(n, heads, dk, seed=i), rnd(n, heads, dk, seed=10 + i, scale=dk ** -0.5), rnd(n, heads, dv, seed=20 + i))
@@ -92,7 +98,7 @@ def test_the_recurrence_in_portions_of_any_size_beside_each_other(heads, dk, dv)
     slot = {"a": 2, "b": 0, "c": 3, "d": 0}  # d takes b's slot when b has finished
     done = {r: 0 for r in lengths}
     got = {r: [] for r in lengths}
-    sizes = [5, 1, 2, 9, 1, 1, 17, 3]
+    sizes = [5, 64, 1, 65, 130, 2, 9, 63, 1, 17] if chunks else [5, 1, 2, 9, 1, 1, 17, 3]
     step = 0
     while any(done[r] < lengths[r] for r in lengths):
         live = [r for r in ("a", "b", "c") if done[r] < lengths[r]]
@@ -113,8 +119,12 @@ def test_the_recurrence_in_portions_of_any_size_beside_each_other(heads, dk, dv)
             slots.append(slot[r])
         proj = dev(torch.cat(rows))
         out = torch.full((proj.shape[0], heads * dv), float("nan"), dtype=torch.float32, device=DEV)
-        ops.decay_scan(out, proj, state, ints(slots), ints(cu), ints(ctx), dev(torch.tensor(decay, dtype=F64)),
-                       col_q=0, col_k=heads * dk, col_v=2 * heads * dk, heads=heads, dk=dk, dv=dv)
+        args = (out, proj, state, ints(slots), ints(cu), ints(ctx), dev(torch.tensor(decay, dtype=F64)))
+        cols = dict(col_q=0, col_k=heads * dk, col_v=2 * heads * dk, heads=heads, dk=dk, dv=dv)
+        if chunks:
+            ops.decay_chunks(*args, max(takes.values()), **cols)
+        else:
+            ops.decay_scan(*args, **cols)
         at = 0
         for r in live:
             got[r].append(out[at: at + takes[r]].cpu())
@@ -181,9 +191,9 @@ def paged(t, k_heads, dk, v_heads, dv, bs, dtype, seed=0, spare=3):
     return k_pool, v_pool, ints(order).reshape(1, need), slots
 
 
-def softmax_attention(h, w, m, eps, dtype, bs, portions=(1000,)):
+def softmax_attention(h, w, m, eps, dtype, bs, portions=(1000,), matrix_cores=False):
     """The engine's kernels on one request that comes in portions: projection by the test, then norm_store and
-    attend_composed per portion over shuffled pages."""
+    attend_composed (or, with `matrix_cores`, attend_composed_mfma) per portion over shuffled pages."""
     from llmserve.ops import library as ops
     from llmserve.parts.attention_composed import bias_by_distance
 
@@ -203,9 +213,14 @@ def softmax_attention(h, w, m, eps, dtype, bs, portions=(1000,)):
                        temp_every=int(m["q_temp"]["every"]), positions=ints(range(a, a + n)), slots=ints(slots[a: a + n]),
                        k_pool=k_pool, v_pool=v_pool, block_size=bs)
         out = torch.full((n, heads * dv), float("nan"), dtype=dtype, device=DEV)
-        ops.attend_composed(out, q, k_pool, v_pool, table, ints([0] * n), ints(range(a, a + n)), heads=heads, kv_heads=kv,
-                            dk=dk, dv=dv, block_size=bs, scale=float(m["scale"]), dist_bias=bias,
-                            gate=p[:, (heads + kv) * dk + kv * dv:])
+        gate = p[:, (heads + kv) * dk + kv * dv:]
+        if matrix_cores:
+            ops.attend_composed_mfma(out, q, k_pool, v_pool, table, ints([0, n]), ints([a + n]), 0, 1, n, heads=heads,
+                                     kv_heads=kv, dk=dk, dv=dv, block_size=bs, scale=float(m["scale"]), dist_bias=bias,
+                                     gate=gate)
+        else:
+            ops.attend_composed(out, q, k_pool, v_pool, table, ints([0] * n), ints(range(a, a + n)), heads=heads,
+                                kv_heads=kv, dk=dk, dv=dv, block_size=bs, scale=float(m["scale"]), dist_bias=bias, gate=gate)
         outs.append(out.cpu())
         a += n
     return torch.cat(outs)
@@ -224,7 +239,7 @@ ATTENTION_CASES = [  # heads, kv_heads, dk, dv, table rows, farthest, every, blo
     (4, 2, 16, 24, 10, 40, 9, 8, 90),
     (3, 3, 8, 8, 4, 17, 2, 4, 50),
     (5, 1, 24, 12, 32, 200, 50, 16, 260),
-    (6, 2, 96, 64, 8, 30, 64, 16, 70),
+    (6, 3, 80, 48, 8, 30, 64, 16, 70),
     (1, 1, 10, 6, 2, 5, 1, 8, 20),
 ]
 
@@ -243,6 +258,30 @@ def test_normed_queries_distance_table_and_gate(dtype, heads, kv, dk, dv, rows, 
     want = pf.gated_softmax_attention(h, w, m, eps)
     close(softmax_attention(h, w, m, eps, dtype, bs), want, dtype, "whole", loose=3)
     close(softmax_attention(h, w, m, eps, dtype, bs, portions=(7, 2, 1, 19, 1, 1)), want, dtype, "in portions", loose=3)
+
+
+MATRIX_CORE_CASES = [  # heads, kv_heads, dk, dv, table rows, farthest, every, block size, tokens
+    (4, 2, 16, 32, 10, 40, 9, 16, 300),    # most keys lie beyond the table's reach
+    (8, 1, 64, 64, 32, 200, 50, 16, 420),  # groups of tiles that the scalar unit addresses
+    (6, 3, 80, 48, 8, 30, 64, 8, 150),
+    (3, 3, 32, 16, 4, 1000, 2, 4, 70),     # every key within the table's reach
+]
+
+
+@pytest.mark.parametrize("heads,kv,dk,dv,rows,farthest,every,bs,t", MATRIX_CORE_CASES)
+def test_distance_table_and_gate_on_the_matrix_cores(heads, kv, dk, dv, rows, farthest, every, bs, t):
+    """The same as above through the bfloat16 kernel on the matrix cores: whole, in portions, and token by token."""
+    width, eps, dtype = 32, 1e-5, torch.bfloat16
+    m = {"heads": heads, "kv_heads": kv, "dim": dk, "vdim": dv, "scale": 0.8 / math.sqrt(dk), "bias_max": farthest,
+         "q_temp": {"coef": 1.5, "every": every}}
+    h, w = rnd(t, width, seed=41), attention_weights(heads, kv, dk, dv, rows, width, seed=51)
+    h, w = h.to(dtype).double(), {k: v.to(dtype).double() for k, v in w.items()}
+    want = pf.gated_softmax_attention(h, w, m, eps)
+    close(softmax_attention(h, w, m, eps, dtype, bs, matrix_cores=True), want, dtype, "whole", loose=3)
+    close(softmax_attention(h, w, m, eps, dtype, bs, portions=(7, 2, 1, 19, 1, 1, 64), matrix_cores=True), want, dtype,
+          "in portions", loose=3)
+    close(softmax_attention(h, w, m, eps, dtype, bs, portions=(t - 40,) + (1,) * 40, matrix_cores=True), want, dtype,
+          "token by token", loose=3)
 
 
 def test_a_key_that_stands_out_at_every_edge_of_the_distance_table():
@@ -362,7 +401,7 @@ def logits_close(got, ref, dtype, what):
         assert over <= max(1, len(err) // 4), f"{what}: {over} of {len(err)} positions are off by more than 0.04 (worst {worst})"
 
 
-MODELS = {"small": (SMALL, 8), "small_b": (SMALL_B, 16), "small_c": (SMALL_C, 4)}
+MODELS = {"small": (SMALL, 8), "small_b": (SMALL_B, 16), "small_c": (SMALL_C, 4), "small_d": (SMALL_D, 16)}
 
 
 @pytest.fixture(scope="module")
