@@ -254,7 +254,7 @@ def felavik_config(size: dict, layers: int, experts: int = 8, top: int = 2) -> d
         if i % 4 == 1:
             entry = {"type": "parallel", "mlp": mlp, "mixer": {
                 "left": {"heads": heads, "kv_heads": size["kv_heads"], "dim": dim, "vdim": dim, "scale": dim ** -0.5,
-                         "bias_max": 1024, "bias_rows": 32, "q_temp": {"coef": 0.1, "every": 1024}},
+                         "bias_max": 128, "bias_rows": 32, "q_temp": {"coef": 0.1, "every": 1024}},
                 "right": {"heads": heads // 2, "dim": dim, "vdim": dim, "decay": decays(heads // 2),
                           "rot": {"base": 10000.0, "dims": dim}},
                 "left_scale": 1.0, "right_scale": 1.0}}

@@ -85,6 +85,13 @@ struct AttnArgs {
     // decoding, every request of the launch with exactly one new token: the row of request seq_begin + i is
     // one_token_from + i, which saves a workgroup the wait for cu_seqlens before it can ask for its queries (-1: not so)
     int one_token_from;
+    // prompts only: a bias per head and distance, [heads, dist_reach + 1] with the last entry for everything beyond,
+    // added to the scaled score (null: none), and 32-bit products [rows, gate_stride] by whose sigmoid the result is
+    // multiplied (null: none)
+    const float* dist_bias;
+    int dist_reach;
+    const float* gate;
+    int gate_stride;
 };
 
 // 2^x by the hardware's own instruction.  Scores are kept in units of log2(e) (scale_log2 = scale * log2 e), so
@@ -137,11 +144,16 @@ __device__ __forceinline__ float column_sum(float x) {
 //   fill_values(): called once the score products are issued, may bring vf in then (it is read after the softmax):
 //   what it asks LDS for arrives while the vector unit is busy, and does not stand in the way of the key rows.
 #define STALE_MAX 8.f  // by how much (in powers of two) a column's maximum may pass the reference before a rescale
-template <int DB, int KS, bool MASKED, int CG, class FillValues>
+//   BIAS: bias_row[min(distance, reach)] (times log2 e) is added to every scaled score, the distance being the
+//   column's position less the key's; `far` is the entry at `reach` times log2 e, which a tile that lies beyond the
+//   reach for every lane takes without a load.  The scores are then scaled at once and the rest works in those units.
+template <int DB, int KS, bool MASKED, int CG, bool BIAS = false, class FillValues>
 __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (&m_run)[CG], float (&l_run)[CG],
                                                    const uint4 (&kf)[2][KS], uint4 (&vf)[DB], const uint4 (&qf)[CG][KS],
-                                                   int jk, const int (&lo_col)[CG], const int (&p_col)[CG], float scale_log2,
-                                                   FillValues fill_values) {
+                                                   int jk, const int (&lo_col)[CG], const int (&p_col)[CG], float scale_log2_in,
+                                                   FillValues fill_values, const float* bias_row = nullptr, int reach = 0,
+                                                   float far = 0.f) {
+    const float scale_log2 = BIAS ? 1.f : scale_log2_in;
     f32x4 s_acc[CG][2];
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg)
@@ -159,6 +171,23 @@ __device__ __forceinline__ void attend_tile_groups(f32x4 (&acc)[CG][DB], float (
 #pragma unroll
     for (int cg = 0; cg < CG; ++cg) {
         float tmax = -INFINITY;
+        if constexpr (BIAS) {
+            const int d0 = p_col[cg] - jk;  // the distance of the lane's first key; the others are nearer by one each
+            if (__builtin_amdgcn_ballot_w64(d0 - 7 < reach) == 0) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s_acc[cg][e / 4][e % 4] = fmaf(s_acc[cg][e / 4][e % 4], scale_log2_in, far);
+            } else {
+                float bias[8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {  // (a key ahead of the column is masked below; its entry is read from a place that exists)
+                    const int d = d0 - e;
+                    bias[e] = bias_row[d < 0 ? 0 : (d < reach ? d : reach)];
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    s_acc[cg][e / 4][e % 4] = fmaf(s_acc[cg][e / 4][e % 4], scale_log2_in, bias[e] * 1.44269504088896341f);
+            }
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             sc[cg][e] = s_acc[cg][e / 4][e % 4];
@@ -551,7 +580,7 @@ __global__ __launch_bounds__(NW* LLMS_WAVE) void attn_mfma_kernel(const AttnArgs
 // a SIMD always has two waves to switch between (four up to head_dim 64, where two workgroups share a CU), and the
 // blocks are handed out in an order (see `rank` below) in which a CU that was given a long one gets a short one
 // beside or after it.
-template <int DB, bool TWIN, int CG, int WB>
+template <int DB, bool TWIN, int CG, int WB, bool BIAS = false>
 __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) ? 4 : 1) void attn_prompt_kernel(const AttnArgs a) {
     constexpr int D = DB * 16;
     constexpr int KS = (D + 31) / 32;
@@ -638,6 +667,9 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
     const bf16* k_base = a.k_pool + (size_t)kvh * a.block_size * D;
     const bf16* v_base = a.v_pool + (size_t)kvh * a.block_size * D;
     const float scale_log2 = a.scale * 1.44269504088896341f;
+    // the column's head's row of the distance table (a column without a head reads the first row and is discarded)
+    const float* bias_row = BIAS ? a.dist_bias + (size_t)(c_head_in < G ? head : 0) * (a.dist_reach + 1) : nullptr;
+    const float bias_far = BIAS ? bias_row[a.dist_reach] * 1.44269504088896341f : 0.f;
     // the tiles whose 32 keys every column of this wave sees: up to the wave's first token, from the window's
     // start of its last one
     const int w_last = min(w_first + CG * TPG, n_new) - 1;
@@ -768,8 +800,8 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
 #pragma unroll
                 for (int m = 0; m < DB; ++m) vf[m] = vt[(16 * m + col) * 4 + g];
             };
-            if (all_seen) attend_tile_groups<DB, KS, false, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values);
-            else attend_tile_groups<DB, KS, true, CG>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values);
+            if (all_seen) attend_tile_groups<DB, KS, false, CG, BIAS>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values, bias_row, a.dist_reach, bias_far);
+            else attend_tile_groups<DB, KS, true, CG, BIAS>(acc, m_run, l_run, kf, vf, qf, j0 + 8 * g, lo_col, p_col, scale_log2, read_values, bias_row, a.dist_reach, bias_far);
         }
         if (TWIN && twin == 0) fetch_ahead();
         __syncthreads();
@@ -834,6 +866,18 @@ __global__ __launch_bounds__((TWIN ? 2 : 1) * WB * LLMS_WAVE, (TWIN && DB <= 4) 
         }
         const float inv = 1.f / l_run[cg];
         bf16* orow = a.out + (size_t)(tok0 + c_tok[cg]) * a.out_stride + (size_t)head * D;
+        if (BIAS && a.gate) {
+            const float* grow = a.gate + (size_t)(tok0 + c_tok[cg]) * a.gate_stride + (size_t)head * D;
+#pragma unroll
+            for (int m = 0; m < DB; ++m) {
+                const float4 z = *reinterpret_cast<const float4*>(grow + 16 * m + 4 * g);
+                uint2 w;
+                w.x = pack_bf16(acc[cg][m][0] * inv / (1.f + expf(-z.x)), acc[cg][m][1] * inv / (1.f + expf(-z.y)));
+                w.y = pack_bf16(acc[cg][m][2] * inv / (1.f + expf(-z.z)), acc[cg][m][3] * inv / (1.f + expf(-z.w)));
+                *reinterpret_cast<uint2*>(orow + 16 * m + 4 * g) = w;
+            }
+            continue;
+        }
 #pragma unroll
         for (int m = 0; m < DB; ++m) {
             uint2 w;
@@ -891,15 +935,15 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(bf16* __restrict__ out,
 
 #define PROMPT_TWIN_MAX_DB 12  // widest head (in blocks of 16 dimensions) whose 8 waves with twins fit the registers
 
-template <int DB, int CG>
+template <int DB, int CG, bool BIAS = false>
 static void launch_prompt_cg(dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
     if constexpr (DB <= PROMPT_TWIN_MAX_DB) {  // (wider heads are never given twins, so those kernels are not built)
         if (twin) {
-            attn_prompt_kernel<DB, true, CG, PROMPT_WB><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+            attn_prompt_kernel<DB, true, CG, PROMPT_WB, BIAS><<<grid, 2 * PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
             return;
         }
     }
-    attn_prompt_kernel<DB, false, CG, PROMPT_WB><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
+    attn_prompt_kernel<DB, false, CG, PROMPT_WB, BIAS><<<grid, PROMPT_WB * LLMS_WAVE, 0, stream>>>(a);
 }
 
 // Few tokens (decoding): small workgroups, so that the merge reaches many CUs; many tokens: 256 threads each.
@@ -910,6 +954,23 @@ static void launch_merge(void* out, int out_stride, const float* ws_o, const flo
         (bf16*)out, out_stride, ws_o, ws_ml, token_begin, n_heads, head_dim, num_splits);
 }
 
+#ifdef LLMS_ATTENTION_BIASED
+// The prompt kernel with a distance table and an output gate, built for heads of 32, 64, 96 and 128.
+static int launch_prompt(int db, int cg, dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
+#define ATT_CASE(N)                                                                       \
+    case N:                                                                               \
+        if (cg == 2 && PROMPT_CG_MAX(N) == 2) launch_prompt_cg<N, PROMPT_CG_MAX(N), true>(grid, twin, a, stream); \
+        else launch_prompt_cg<N, 1, true>(grid, twin, a, stream);                       \
+        break;
+    switch (db) {
+        ATT_CASE(2) ATT_CASE(4) ATT_CASE(6) ATT_CASE(8)
+        default:
+            LLMS_REQUIRE(false, "attention_mfma: with a distance table head_dim is 32, 64, 96 or 128");
+    }
+#undef ATT_CASE
+    return LLMS_OK;
+}
+#else
 static int launch_prompt(int db, int cg, dim3 grid, bool twin, const AttnArgs& a, hipStream_t stream) {
 #define ATT_CASE(N)                                                                       \
     case N:                                                                               \
@@ -925,6 +986,8 @@ static int launch_prompt(int db, int cg, dim3 grid, bool twin, const AttnArgs& a
 #undef ATT_CASE
     return LLMS_OK;
 }
+
+#endif
 
 // CUs of the current device (asked once per device).
 static int compute_units(int* out) {
@@ -942,6 +1005,11 @@ static int compute_units(int* out) {
     return LLMS_OK;
 }
 
+#ifdef LLMS_ATTENTION_BIASED
+static int launch_attn(int, dim3, int, const AttnArgs&, hipStream_t) {
+    LLMS_REQUIRE(false, "attention_mfma: the kernel with a distance table takes portions of prompts only");
+}
+#else
 static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStream_t stream) {
 #define ATT_CASE(N)                                                                                  \
     case N:                                                                                          \
@@ -958,6 +1026,8 @@ static int launch_attn(int db, dim3 grid, int threads, const AttnArgs& a, hipStr
     return LLMS_OK;
 }
 
+#endif
+
 extern "C" {
 
 // Attention for the requests [seq_begin, seq_begin + n_seqs) of a step.  max_new: most new tokens any of
@@ -968,13 +1038,14 @@ extern "C" {
 // ws_ml [tokens * heads * splits * 2] floats, indexed by absolute token row.  `arrive` (may be null): n_arrive
 // counters in device memory, all zero, which the kernel leaves zero: decoding with 2 to 16 splits then adds the
 // shares up in the workgroup that finishes last instead of in a second kernel.
-int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+static int attention_mfma_launch(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
                         const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
                         const int* cu_seqlens,
                         const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
                         int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
                         float scale, int split_waves, int num_splits, int waves, float* ws_o, float* ws_ml,
-                        unsigned* arrive, int n_arrive, hipStream_t stream) {
+                        unsigned* arrive, int n_arrive, const float* dist_bias, int dist_reach, const float* gate,
+                        int gate_stride, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && n_heads > 0 && n_kv_heads > 0, "attention_mfma: sizes must be positive");
     LLMS_REQUIRE(n_heads % n_kv_heads == 0, "attention_mfma: n_heads must be a multiple of n_kv_heads");
     LLMS_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256, "attention_mfma: head_dim must be a multiple of 16 up to 256");
@@ -997,7 +1068,8 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     const int groups = (max_new + TPG - 1) / TPG;
     AttnArgs a = {(bf16*)out, out_stride, (const bf16*)q, q_stride, (const bf16*)k_pool, (const bf16*)v_pool,
                   block_tables, table_rows, max_blocks, cu_seqlens, context_lens, seq_begin, n_heads, n_kv_heads, block_size,
-                  window, scale, num_splits, ws_o, ws_ml, nullptr, token_begin + n_tokens, 0, -1};
+                  window, scale, num_splits, ws_o, ws_ml, nullptr, token_begin + n_tokens, 0, -1,
+                  dist_bias, dist_reach, gate, gate_stride};
     // (at most one token each and as many tokens as requests: every request has exactly one, in the order of the requests)
     if (split_waves > 0 && max_new == 1 && n_tokens == n_seqs) a.one_token_from = token_begin;
     LLMS_REQUIRE(n_kv_heads * HB <= 65535, "attention_mfma: too many heads");
@@ -1054,7 +1126,44 @@ int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, 
     LLMS_LAUNCH_CHECK();
 }
 
+#ifndef LLMS_ATTENTION_BIASED
+// The plain attention: no distance table, no gate.
+int llms_attention_mfma(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+                        const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                        const int* cu_seqlens,
+                        const int* context_lens, int seq_begin, int n_seqs, int max_new, int token_begin,
+                        int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size, int window,
+                        float scale, int split_waves, int num_splits, int waves, float* ws_o, float* ws_ml,
+                        unsigned* arrive, int n_arrive, hipStream_t stream) {
+    return attention_mfma_launch(out, out_stride, q, q_stride, k_pool, v_pool, block_tables, table_rows, max_blocks, cu_seqlens,
+                                 context_lens, seq_begin, n_seqs, max_new, token_begin, n_tokens, n_heads, n_kv_heads, head_dim,
+                                 block_size, window, scale, split_waves, num_splits, waves, ws_o, ws_ml, arrive, n_arrive,
+                                 nullptr, 0, nullptr, 0, stream);
+}
+#else
+// Prompt portions with a bias per head and distance on the scaled scores (dist_bias float [n_heads, dist_reach + 1],
+// the last entry for every distance beyond) and, optionally, the result multiplied by the sigmoid of 32-bit gate
+// products [rows, gate_stride] (16-byte aligned rows).  Heads of 32, 64, 96 or 128 numbers; no window, no splits.
+int llms_attention_prompt_biased(void* out, int out_stride, const void* q, int q_stride, const void* k_pool,
+                                 const void* v_pool, const int* block_tables, const int* table_rows, int max_blocks,
+                                 const int* cu_seqlens, const int* context_lens, int seq_begin, int n_seqs, int max_new,
+                                 int token_begin, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int block_size,
+                                 float scale, const float* dist_bias, int dist_reach, const float* gate, int gate_stride,
+                                 hipStream_t stream) {
+    LLMS_REQUIRE(dist_bias && dist_reach >= 0, "attention_prompt_biased: a distance table with at least one entry per head");
+    LLMS_REQUIRE(head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128,
+                 "attention_prompt_biased: head_dim is 32, 64, 96 or 128");
+    LLMS_REQUIRE(!gate || (gate_stride % 4 == 0 && ((uintptr_t)gate % 16) == 0), "attention_prompt_biased: gate rows must be 16-byte aligned");
+    return attention_mfma_launch(out, out_stride, q, q_stride, k_pool, v_pool, block_tables, table_rows, max_blocks, cu_seqlens,
+                                 context_lens, seq_begin, n_seqs, max_new, token_begin, n_tokens, n_heads, n_kv_heads, head_dim,
+                                 block_size, /*window=*/0, scale, /*split_waves=*/0, /*num_splits=*/1, /*waves=*/4, nullptr,
+                                 nullptr, nullptr, 0, dist_bias, dist_reach, gate, gate_stride, stream);
+}
+#endif
+
 }  // extern "C"
+
+#ifndef LLMS_ATTENTION_BIASED
 
 // ---------------------------------------------------------------------------------------------------------
 // Decoding with the keys of a request shared out to several workgroups, without a workspace from the caller:
@@ -1118,3 +1227,4 @@ int llms_attention_decode_noalloc(void* out, int out_stride, const void* q, int 
 }
 
 }  // extern "C"
+#endif  // LLMS_ATTENTION_BIASED

@@ -733,6 +733,53 @@ def attention_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_p
     return out
 
 
+def attention_prompt_biased_supported(dtype: torch.dtype, dk: int, dv: int, block_size: int) -> bool:
+    """Whether `attention_prompt_biased` takes this cache: bfloat16, keys and values of one size, 32, 64, 96 or 128."""
+    return dtype == torch.bfloat16 and dk == dv and dk in (32, 64, 96, 128) and block_size % 8 == 0
+
+
+def attention_prompt_biased(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                            block_tables: torch.Tensor, cu_seqlens: torch.Tensor, context_lens: torch.Tensor,
+                            seq_begin: int, n_seqs: int, max_new: int, token_begin: int, n_tokens: int, *, n_heads: int,
+                            n_kv_heads: int, head_dim: int, block_size: int, scale: float, dist_bias: torch.Tensor,
+                            gate: torch.Tensor | None = None, table_rows: torch.Tensor | None = None) -> torch.Tensor:
+    """The prompt kernel of `attention_mfma` (no window, no splits) with dist_bias[h, min(i - j, R)] added to the scaled
+    score of head h between positions i >= j (float32 [heads, R + 1]) and, with `gate` (float32 [N, >= heads * head_dim],
+    16-byte aligned rows), the result multiplied by the sigmoid of the gate's products."""
+    dev = _dev(out, q, k_pool, v_pool, block_tables, cu_seqlens, context_lens, table_rows, dist_bias, gate)
+    _check_paged(q, out, k_pool, v_pool, block_tables, n_heads, n_kv_heads, head_dim, block_size)
+    if not attention_prompt_biased_supported(q.dtype, head_dim, head_dim, block_size):
+        raise ValueError("attention_prompt_biased needs bfloat16, heads of 32, 64, 96 or 128 and pages of a multiple of 8 keys")
+    b = cu_seqlens.numel() - 1
+    _i32(cu_seqlens, "cu_seqlens")
+    _i32(context_lens, "context_lens", b)
+    if table_rows is not None:
+        _i32(table_rows, "table_rows", b)
+    elif block_tables.shape[0] < b:
+        raise ValueError("block_tables has fewer rows than there are requests")
+    if not (0 <= seq_begin and n_seqs >= 0 and seq_begin + n_seqs <= b):
+        raise ValueError("request range is outside the batch")
+    if not (0 <= token_begin and token_begin + n_tokens <= q.shape[0]):
+        raise ValueError("token range is outside the batch")
+    if q.stride(0) % 8 or q.data_ptr() % 16 or out.data_ptr() % 16:
+        raise ValueError("q rows must be 16-byte aligned")
+    if dist_bias.dtype != torch.float32 or dist_bias.dim() != 2 or dist_bias.shape[0] != n_heads or dist_bias.shape[1] < 1 \
+            or not dist_bias.is_contiguous():
+        raise ValueError("dist_bias must be a contiguous float32 [heads, reach + 1] tensor")
+    if gate is not None and (gate.dtype != torch.float32 or gate.dim() != 2 or gate.stride(1) != 1 or gate.shape[0] != q.shape[0]
+                             or gate.shape[1] < n_heads * head_dim or gate.stride(0) % 4 or gate.data_ptr() % 16):
+        raise ValueError("gate must be float32 [N, >= heads*head_dim] with unit inner stride and 16-byte aligned rows")
+    if n_seqs == 0 or n_tokens == 0:
+        return out
+    _check(load("attention_biased").llms_attention_prompt_biased(
+        _ptr(out), c_int(out.stride(0)), _ptr(q), c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
+        _ptr(table_rows), c_int(block_tables.shape[1]), _ptr(cu_seqlens), _ptr(context_lens), c_int(seq_begin), c_int(n_seqs),
+        c_int(max_new), c_int(token_begin), c_int(n_tokens), c_int(n_heads), c_int(n_kv_heads), c_int(head_dim),
+        c_int(block_size), c_float(scale), _ptr(dist_bias), c_int(dist_bias.shape[1] - 1), _ptr(gate),
+        c_int(gate.stride(0) if gate is not None else 0), _stream(dev)), "attention_prompt_biased")
+    return out
+
+
 # ------------------------------------------------------------------------------ a residual stream in 32-bit
 
 

@@ -148,7 +148,19 @@ class ComposedAttention(Mixer):
         self.lam = 0.0
 
     def libraries(self, dtype_name):
-        return ("attention_composed", "attention_composed_mfma") if dtype_name == "bfloat16" else ("attention_composed",)
+        if dtype_name != "bfloat16":
+            return ("attention_composed",)
+        names = ("attention_composed", "attention_composed_mfma")
+        return names + ("attention_biased",) if self.plain_but_for_bias_and_gate else names
+
+    @property
+    def plain_but_for_bias_and_gate(self) -> bool:
+        """One score map over every earlier key, with nothing between the scores and the values but a distance table,
+        and nothing behind them but a gate: what the prompt kernel of the plain attention takes in its variant with a
+        table (keys and values of one size of 32, 64, 96 or 128)."""
+        return (self.rel_rows > 0 and self.maps == 1 and self.window is None and self.chunk is None and not self.talking
+                and self.slope_base is None and self.head_norm_eps is None and self.head_dim == self.value_dim
+                and self.head_dim in (32, 64, 96, 128))
 
     # ---- what it keeps between steps -------------------------------------------------------------
     def cache_spec(self):
@@ -278,6 +290,16 @@ class ComposedAttention(Mixer):
         if n_dec:
             ops.attend_composed_mfma(*args, 0, n_dec, 1, shares=self.decode_shares(n_dec, batch.max_decode_context,
                                                                                   ops.compute_units(q.device)), **common)
+        if n_dec < batch.num_seqs and self.plain_but_for_bias_and_gate and \
+                ops.attention_prompt_biased_supported(q.dtype, self.head_dim, self.value_dim, paged.block_size) and \
+                (gate is None or (gate.data_ptr() % 16 == 0 and gate.stride(0) % 4 == 0)) and q.stride(0) % 8 == 0:
+            # portions of prompts: the plain attention's kernel (keys and values shared by a workgroup's waves through LDS)
+            ops.attention_prompt_biased(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens,
+                                        batch.context_lens, n_dec, batch.num_seqs - n_dec, batch.max_count, n_dec,
+                                        batch.num_tokens - n_dec, n_heads=self.num_heads, n_kv_heads=self.num_kv_heads,
+                                        head_dim=self.head_dim, block_size=paged.block_size, scale=self.scale,
+                                        dist_bias=self.dist_bias, gate=gate, table_rows=batch.state_slots)
+            return
         if n_dec < batch.num_seqs:
             shares = self.prompt_shares(batch.num_seqs - n_dec, batch.max_count, batch.max_context,
                                         ops.compute_units(q.device))

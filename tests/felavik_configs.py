@@ -79,6 +79,9 @@ def _small_d():
                        right={"heads": 2, "dim": 32, "vdim": 16, "decay": [0.9, 0.999], "rot": {"base": 1000.0, "dims": 16}}),
               lightning(heads=1, dim=64, vdim=32, decay=[0.98], mlp=moe(4, 2, 32, 2, 1))]
     layers.append(again(layers, 1))
+    # keys and values of one size: portions of prompts take the plain attention's kernel with a table
+    layers.append(parallel(left={"heads": 2, "kv_heads": 1, "dim": 32, "vdim": 32, "bias_max": 20, "bias_rows": 6,
+                                 "q_temp": {"coef": 0.3, "every": 7}}, mlp=None))
     return config_of(layers, width=64, vocab=173, scale=1.2)
 
 

@@ -214,7 +214,11 @@ def softmax_attention(h, w, m, eps, dtype, bs, portions=(1000,), matrix_cores=Fa
                        k_pool=k_pool, v_pool=v_pool, block_size=bs)
         out = torch.full((n, heads * dv), float("nan"), dtype=dtype, device=DEV)
         gate = p[:, (heads + kv) * dk + kv * dv:]
-        if matrix_cores:
+        if matrix_cores == "prompt":
+            ops.attention_prompt_biased(out, q, k_pool, v_pool, table, ints([0, n]), ints([a + n]), 0, 1, n, 0, n, n_heads=heads,
+                                        n_kv_heads=kv, head_dim=dk, block_size=bs, scale=float(m["scale"]), dist_bias=bias,
+                                        gate=gate)
+        elif matrix_cores:
             ops.attend_composed_mfma(out, q, k_pool, v_pool, table, ints([0, n]), ints([a + n]), 0, 1, n, heads=heads,
                                      kv_heads=kv, dk=dk, dv=dv, block_size=bs, scale=float(m["scale"]), dist_bias=bias,
                                      gate=gate)
@@ -282,6 +286,29 @@ def test_distance_table_and_gate_on_the_matrix_cores(heads, kv, dk, dv, rows, fa
           "in portions", loose=3)
     close(softmax_attention(h, w, m, eps, dtype, bs, portions=(t - 40,) + (1,) * 40, matrix_cores=True), want, dtype,
           "token by token", loose=3)
+
+
+PROMPT_KERNEL_CASES = [  # heads, kv_heads, head size, table rows, farthest, every, block size, tokens
+    (8, 1, 64, 32, 200, 50, 16, 420),
+    (4, 2, 32, 10, 40, 9, 8, 300),     # most keys lie beyond the table's reach
+    (6, 3, 96, 8, 30, 64, 16, 150),
+    (2, 2, 128, 12, 1000, 5, 32, 200),  # every key within the table's reach
+]
+
+
+@pytest.mark.parametrize("heads,kv,d,rows,farthest,every,bs,t", PROMPT_KERNEL_CASES)
+def test_distance_table_and_gate_in_the_prompt_kernel(heads, kv, d, rows, farthest, every, bs, t):
+    """The plain attention's prompt kernel in its variant with a distance table and a gate: whole, and in portions
+    behind what the earlier portions left in the pages."""
+    width, eps, dtype = 32, 1e-5, torch.bfloat16
+    m = {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": 0.8 / math.sqrt(d), "bias_max": farthest,
+         "q_temp": {"coef": 1.5, "every": every}}
+    h, w = rnd(t, width, seed=42), attention_weights(heads, kv, d, d, rows, width, seed=52)
+    h, w = h.to(dtype).double(), {k: v.to(dtype).double() for k, v in w.items()}
+    want = pf.gated_softmax_attention(h, w, m, eps)
+    close(softmax_attention(h, w, m, eps, dtype, bs, matrix_cores="prompt"), want, dtype, "whole", loose=3)
+    close(softmax_attention(h, w, m, eps, dtype, bs, portions=(70, 2, 33, 19, 64, 5), matrix_cores="prompt"), want, dtype,
+          "in portions", loose=3)
 
 
 def test_a_key_that_stands_out_at_every_edge_of_the_distance_table():
