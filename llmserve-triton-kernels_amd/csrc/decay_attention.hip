@@ -64,11 +64,20 @@ __global__ __launch_bounds__(DA_THREADS) void decay_prepare_kernel(
 }
 
 // grid: (ceil(dv / 64), heads, requests).  Thread (r, j): column 64 * slice + j, rows r, r + 4, ... (RPT of them).
-template <int RPT>
+// PREP: q, k and v are taken as the projection left them, and what decay_prepare would do to them (activation, rotation
+// by positions[row], the factor on k) is done on their way in, with the same arithmetic; proj is not written.
+struct DecayPrep {
+    const int* positions;
+    const float* freq;
+    int rot_dims, act;
+    float key_scale;
+};
+
+template <int RPT, bool PREP>
 __global__ __launch_bounds__(DA_THREADS) void decay_scan_kernel(
     float* __restrict__ out, int out_stride, const float* __restrict__ proj, int stride, int col_q, int col_k, int col_v,
     float* __restrict__ state, const int* __restrict__ state_slots, const int* __restrict__ cu_seqlens,
-    const int* __restrict__ context_lens, const float* __restrict__ decay, int heads, int dk, int dv) {
+    const int* __restrict__ context_lens, const float* __restrict__ decay, int heads, int dk, int dv, const DecayPrep prep) {
     __shared__ float qk[2][4 * RPT * 2];
     __shared__ float part[2][DA_ROWGROUPS][DA_COLS];
     const int b = blockIdx.z, h = blockIdx.y;
@@ -91,9 +100,29 @@ __global__ __launch_bounds__(DA_THREADS) void decay_scan_kernel(
     for (int t = 0; t < count; ++t) {
         const float* row = proj + (size_t)(row0 + t) * stride;
         float* buf = qk[t & 1];
-        for (int i = threadIdx.x; i < 2 * dk; i += DA_THREADS)
-            buf[i] = i < dk ? row[col_q + h * dk + i] : row[col_k + h * dk + (i - dk)];
-        const float v = c < dv ? row[col_v + h * dv + c] : 0.f;
+        for (int i = threadIdx.x; i < 2 * dk; i += DA_THREADS) {
+            const bool key = i >= dk;
+            const int e = key ? i - dk : i;
+            const float* src = row + (key ? col_k : col_q) + h * dk;
+            float x = src[e];
+            if constexpr (PREP) {
+                if (prep.act == DA_ACT_SILU) x = da_silu(x);
+                if (e < prep.rot_dims) {  // dimension e < half is turned together with dimension e + half
+                    const int half = prep.rot_dims / 2;
+                    const bool first = e < half;
+                    float y = src[first ? e + half : e - half];
+                    if (prep.act == DA_ACT_SILU) y = da_silu(y);
+                    const float2 sc = rotary_angle((float)prep.positions[row0 + t], prep.freq[first ? e : e - half]);
+                    const float2 turned = first ? rotate_pair(x, y, sc.y, sc.x) : rotate_pair(y, x, sc.y, sc.x);
+                    x = first ? turned.x : turned.y;
+                }
+                if (key) x *= prep.key_scale;
+            }
+            buf[i] = x;
+        }
+        float v = c < dv ? row[col_v + h * dv + c] : 0.f;
+        if constexpr (PREP)
+            if (prep.act == DA_ACT_SILU) v = da_silu(v);
         __syncthreads();
         // (the sums of the token before, left in the other buffer, are added up behind this barrier)
         if (t > 0 && r == 0 && c < dv) {
@@ -356,16 +385,33 @@ int llms_decay_prepare(float* proj, int stride, int col_q, int col_k, int col_v,
     LLMS_LAUNCH_CHECK();
 }
 
+// `prepare` != 0: the rows of proj are as the projection left them, and positions, freq, rot_dims, act and key_scale say
+// what llms_decay_prepare would have done to them (done here on their way in; proj is left as it is).
 int llms_decay_scan(float* out, int out_stride, const float* proj, int stride, int col_q, int col_k, int col_v, float* state,
                     const int* state_slots, const int* cu_seqlens, const int* context_lens, const float* decay, int n_seqs,
-                    int heads, int dk, int dv, hipStream_t stream) {
+                    int heads, int dk, int dv, int prepare, const int* positions, const float* freq, int rot_dims, int act,
+                    float key_scale, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && heads > 0 && dk > 0 && dv > 0, "decay_scan: sizes must be positive");
     LLMS_REQUIRE(dk <= 256, "decay_scan: keys of up to 256 numbers");
     LLMS_REQUIRE(heads <= 65535 && n_seqs <= 65535, "decay_scan: up to 65,535 heads and requests");
+    if (prepare) {
+        LLMS_REQUIRE(rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0, "decay_scan: an even number of turned dimensions, up to dk");
+        LLMS_REQUIRE(rot_dims == 0 || (freq && positions), "decay_scan: a rotation needs frequencies and positions");
+        LLMS_REQUIRE(act == DA_ACT_NONE || act == DA_ACT_SILU, "decay_scan: activation 0 (none) or 1 (SiLU)");
+    }
+    const DecayPrep prep = {positions, freq, rot_dims, act, key_scale};
     dim3 grid((dv + DA_COLS - 1) / DA_COLS, heads, n_seqs);
-#define DA_GO(RPT)                                                                                                     \
-    decay_scan_kernel<RPT><<<grid, DA_THREADS, 0, stream>>>(out, out_stride, proj, stride, col_q, col_k, col_v, state,  \
-                                                            state_slots, cu_seqlens, context_lens, decay, heads, dk, dv)
+#define DA_GO(RPT)                                                                                                          \
+    do {                                                                                                                    \
+        if (prepare)                                                                                                        \
+            decay_scan_kernel<RPT, true><<<grid, DA_THREADS, 0, stream>>>(out, out_stride, proj, stride, col_q, col_k, col_v, \
+                                                                          state, state_slots, cu_seqlens, context_lens,     \
+                                                                          decay, heads, dk, dv, prep);                      \
+        else                                                                                                                \
+            decay_scan_kernel<RPT, false><<<grid, DA_THREADS, 0, stream>>>(out, out_stride, proj, stride, col_q, col_k,     \
+                                                                           col_v, state, state_slots, cu_seqlens,           \
+                                                                           context_lens, decay, heads, dk, dv, prep);       \
+    } while (0)
     if (dk <= 32) DA_GO(8);
     else if (dk <= 64) DA_GO(16);
     else if (dk <= 128) DA_GO(32);

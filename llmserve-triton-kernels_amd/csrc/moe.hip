@@ -212,6 +212,54 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_scatter_kernel(
     for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = from_f32<T>(wgt * to_f32(src[c]));
 }
 
+// Few pairs (decoding): the sort and the scatter in one launch.  grid: pairs; dynamic LDS: experts ints (used by the first
+// workgroup).  Every workgroup reads all choices and counts, for its own pair p of expert e, the pairs of experts before e
+// and the earlier pairs of e itself: their sum is the pair's row in the order sorted stably by expert, the same row as
+// moe_rank, moe_offsets and moe_scatter give.  The first workgroup also counts every expert's pairs and leaves seg and
+// tile_start.
+template <typename T>
+__global__ __launch_bounds__(MOE_THREADS) void moe_place_few_kernel(
+    T* __restrict__ xs, int* __restrict__ place, int* __restrict__ seg, int* __restrict__ tile_start, const T* __restrict__ h,
+    const int* __restrict__ chosen, const float* __restrict__ weight, int pairs, int hidden, int top, int experts, int tile_a,
+    int tile_b) {
+    extern __shared__ int hist[];
+    __shared__ float red[16];
+    const int p = blockIdx.x, n = p / top, e = chosen[p];
+    int ahead = 0;
+    for (int q = threadIdx.x; q < pairs; q += MOE_THREADS) {
+        const int c = chosen[q];
+        ahead += (c < e || (c == e && q < p)) ? 1 : 0;
+    }
+    const int dest = (int)block_sum((float)ahead, red);  // (whole numbers far below 2^24: exact)
+    if (threadIdx.x == 0) place[p] = dest;
+    const T* src = h + (size_t)n * hidden;
+    T* dst = xs + (size_t)dest * hidden;
+    if (!weight) {
+        for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = src[c];
+    } else {
+        const float wgt = weight[p];
+        for (int c = threadIdx.x; c < hidden; c += MOE_THREADS) dst[c] = from_f32<T>(wgt * to_f32(src[c]));
+    }
+    if (p != 0) return;
+    for (int i = threadIdx.x; i < experts; i += MOE_THREADS) hist[i] = 0;
+    __syncthreads();
+    for (int q = threadIdx.x; q < pairs; q += MOE_THREADS) atomicAdd(&hist[chosen[q]], 1);
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+    int rows = 0, tiles_a = 0, tiles_b = 0;
+    for (int i = 0; i < experts; ++i) {
+        seg[i] = rows;
+        tile_start[i] = tiles_a;
+        tile_start[experts + 1 + i] = tiles_b;
+        rows += hist[i];
+        tiles_a += (hist[i] + tile_a - 1) / tile_a;
+        tiles_b += (hist[i] + tile_b - 1) / tile_b;
+    }
+    seg[experts] = rows;
+    tile_start[experts] = tiles_a;
+    tile_start[2 * experts + 1] = tiles_b;
+}
+
 // grid: tokens.  rows [parts, pairs, hidden]: a choice's result may arrive as several partial sums
 __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ rows,
                                                                   const int* __restrict__ place, int hidden, int top,
@@ -299,6 +347,24 @@ int llms_moe_scatter(int dtype, void* xs, int* place, const void* h, const int* 
     else
         moe_scatter_kernel<bf16><<<pairs, MOE_THREADS, 0, stream>>>((bf16*)xs, place, (const bf16*)h, chosen, weight, rank, seg,
                                                                     hidden, top);
+    LLMS_LAUNCH_CHECK();
+}
+
+// seg [E + 1], tile_start [2, E + 1], place [pairs], xs [pairs, hidden]: llms_moe_sort and llms_moe_scatter in one launch,
+// for up to 2,048 pairs.
+int llms_moe_place_few(int dtype, void* xs, int* place, int* seg, int* tile_start, const void* h, const int* chosen,
+                       const float* weight, int pairs, int hidden, int top, int experts, int tile_a, int tile_b,
+                       hipStream_t stream) {
+    LLMS_REQUIRE(pairs > 0 && pairs <= 2048 && hidden > 0 && top > 0, "moe_place_few: 1 to 2,048 pairs");
+    LLMS_REQUIRE(experts > 0 && experts <= 8192 && tile_a > 0 && tile_b > 0, "moe_place_few: up to 8,192 experts");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "moe_place_few: dtype must be 0 (float32) or 1 (bfloat16)");
+    const size_t lds = (size_t)experts * sizeof(int);
+    if (dtype == 0)
+        moe_place_few_kernel<float><<<pairs, MOE_THREADS, lds, stream>>>((float*)xs, place, seg, tile_start, (const float*)h,
+                                                                         chosen, weight, pairs, hidden, top, experts, tile_a, tile_b);
+    else
+        moe_place_few_kernel<bf16><<<pairs, MOE_THREADS, lds, stream>>>((bf16*)xs, place, seg, tile_start, (const bf16*)h, chosen,
+                                                                        weight, pairs, hidden, top, experts, tile_a, tile_b);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -348,10 +348,13 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
     for (int c4 = threadIdx.x; c4 < n4; c4 += S32_THREADS) {
         const float4 u = *reinterpret_cast<const float4*>(u_row + 4 * c4);
         const float4 w4 = at(weight + 4 * c4);
-        orow[4 * c4 + 0] = from_f32<T>((u.x - mean) * inv * w4.x);
-        orow[4 * c4 + 1] = from_f32<T>((u.y - mean) * inv * w4.y);
-        orow[4 * c4 + 2] = from_f32<T>((u.z - mean) * inv * w4.z);
-        orow[4 * c4 + 3] = from_f32<T>((u.w - mean) * inv * w4.w);
+        const float a = (u.x - mean) * inv * w4.x, b = (u.y - mean) * inv * w4.y;
+        const float c = (u.z - mean) * inv * w4.z, d = (u.w - mean) * inv * w4.w;
+        if constexpr (sizeof(T) == 2) {  // (rows of a multiple of 4 at an aligned start: 8 bytes at once)
+            *reinterpret_cast<uint2*>(orow + 4 * c4) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+        } else {
+            *reinterpret_cast<float4*>(orow + 4 * c4) = make_float4(a, b, c, d);
+        }
     }
 }
 
@@ -467,7 +470,7 @@ int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, in
     LLMS_REQUIRE((size_t)hidden * 4 <= 96 * 1024, "streams_norm: a row of up to 24,576 elements");
     const size_t lds = (size_t)hidden * sizeof(float);
     auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
-    const bool vec = hidden % 4 == 0 && aligned(x_dst) && aligned(x_src) && aligned(y) && aligned(weight);
+    const bool vec = hidden % 4 == 0 && aligned(x_dst) && aligned(x_src) && aligned(y) && aligned(weight) && aligned(out);
 #define STREAMS_GO(KERNEL, T)                                                                                               \
     do {                                                                                                                    \
         if (lds > 32 * 1024)                                                                                                \

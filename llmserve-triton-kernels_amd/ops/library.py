@@ -1643,6 +1643,34 @@ def moe_sort(chosen: torch.Tensor, experts: int):
     return rank, seg, tiles
 
 
+MOE_FEW_PAIRS = 512  # pairs (token, choice) up to which `moe_place_few` sorts and scatters in one launch
+
+
+def moe_place_few(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor, weight: torch.Tensor | None,
+                  experts: int):
+    """`moe_sort` and `moe_scatter` in one launch for few pairs: returns (seg [E + 1], tile_start [2, E + 1]) and fills
+    xs and place as they do (the same rows: sorted by expert, stably)."""
+    dev = _dev(xs, place, h, chosen, weight)
+    _rows(h, "h")
+    _i32(chosen, "chosen")
+    pairs = chosen.numel()
+    _rows(xs, "xs", h.shape[1])
+    top = pairs // max(h.shape[0], 1)
+    if xs.shape[0] != pairs or xs.dtype != h.dtype or top * h.shape[0] != pairs:
+        raise ValueError("xs has a row per pair, in h's dtype")
+    if not 0 < pairs <= 2048:
+        raise ValueError("1 to 2,048 pairs")
+    _i32(place, "place", pairs)
+    if weight is not None:
+        _f32(weight, "weight", pairs)
+    work = torch.empty(3 * experts + 3, dtype=torch.int32, device=dev)
+    seg, tiles = work[: experts + 1], work[experts + 1:]
+    _check(load("moe").llms_moe_place_few(c_int(_code(h)), _ptr(xs), _ptr(place), _ptr(seg), _ptr(tiles), _ptr(h), _ptr(chosen),
+                                          _ptr(weight), c_int(pairs), c_int(h.shape[1]), c_int(top), c_int(experts),
+                                          c_int(GROUPED_TILE), c_int(GROUPED_TILE_MFMA), _stream(dev)), "moe_place_few")
+    return seg, tiles
+
+
 def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: torch.Tensor,
                 weight: torch.Tensor | None, rank: torch.Tensor, seg: torch.Tensor) -> None:
     """xs[seg[chosen[p]] + rank[p]] = weight[p] * h[p // top] (rounded to xs's dtype; `weight` None: the row as it
@@ -1740,14 +1768,27 @@ def _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk,
 
 def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
                cu_seqlens: torch.Tensor, context_lens: torch.Tensor, decay: torch.Tensor, *, col_q: int, col_k: int,
-               col_v: int, heads: int, dk: int, dv: int) -> torch.Tensor:
+               col_v: int, heads: int, dk: int, dv: int, prepare: dict | None = None) -> torch.Tensor:
     """The recurrence S_t = decay_h S_(t-1) + k_t v_t^T, o_t = S_t^T q_t over the new tokens of every request, token by
     token: request b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of proj (float32; q, k, v from the given columns on),
     starts from state[state_slots[b]] (float32 [slots, heads, dk, dv]; from zero when its portion starts at position 0,
     which context_lens[b], its length after the step, tells) and leaves its last state there.  out float32 [N, heads*dv].
-    A request of length 0 is padding: its rows give zeros and no state is touched."""
+    A request of length 0 is padding: its rows give zeros and no state is touched.  `prepare` (the keyword arguments of
+    `decay_prepare`: activation, freq, rot_dims, positions, key_scale): proj is as the projection left it, and what
+    `decay_prepare` would do to q, k and v is done on their way in, with the same arithmetic (proj is not written)."""
     dev = _dev(out, proj, state, state_slots, cu_seqlens, context_lens, decay)
     _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
+    prep = prepare or {}
+    p_positions, p_freq, p_rot = prep.get("positions"), prep.get("freq"), int(prep.get("rot_dims") or 0)
+    if prepare is not None:
+        if prep.get("activation") not in (None, "none", "silu"):
+            raise ValueError(f"activation {prep.get('activation')!r}")
+        if p_rot % 2 or not 0 <= p_rot <= dk:
+            raise ValueError("rot_dims must be even and at most dk")
+        if p_rot:
+            _f32(p_freq, "freq", p_rot // 2)
+            _i32(p_positions, "positions", proj.shape[0])
+            _dev(out, p_freq, p_positions)
     if out.dtype != torch.float32 or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (proj.shape[0], heads * dv):
         raise ValueError(f"out must be float32 [{proj.shape[0]}, {heads * dv}] with unit inner stride")
     if dk > DECAY_MAX_KEY:
@@ -1758,7 +1799,9 @@ def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state
     _check(load("decay_attention").llms_decay_scan(
         _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
         _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), c_int(b), c_int(heads), c_int(dk),
-        c_int(dv), _stream(dev)), "decay_scan")
+        c_int(dv), c_int(0 if prepare is None else 1), _ptr(p_positions if p_rot else None), _ptr(p_freq if p_rot else None),
+        c_int(p_rot), c_int(_ACTIVATIONS[prep.get("activation")] if prepare is not None else 0),
+        c_float(float(prep.get("key_scale", 1.0))), _stream(dev)), "decay_scan")
     return out
 
 

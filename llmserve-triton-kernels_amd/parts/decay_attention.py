@@ -102,21 +102,28 @@ class DecayAttention(Mixer):
         heads, dk, dv = self.num_heads, self.head_dim, self.value_dim
         proj = linear(x, self.in_weight, out_dtype=torch.float32)
         cols = dict(col_q=0, col_k=self.cq, col_v=2 * self.cq, heads=heads, dk=dk, dv=dv)
+        prepare = None
         if self.activation is not None or self.rot_dims or self.key_scale != 1.0:
-            ops.decay_prepare(proj, activation=self.activation, freq=self.freq, rot_dims=self.rot_dims,
-                              positions=batch.positions, key_scale=self.key_scale, **cols)
+            prepare = dict(activation=self.activation, freq=self.freq, rot_dims=self.rot_dims, positions=batch.positions,
+                           key_scale=self.key_scale)
         o = torch.empty((proj.shape[0], self.cv), dtype=torch.float32, device=x.device)
-        self.recur(o, proj, cache.state, batch, cols)
+        self.recur(o, proj, cache.state, batch, cols, prepare)
         out = torch.empty((proj.shape[0], self.cv), dtype=x.dtype, device=x.device)
         ops.decay_finish(out, o, heads=heads, dv=dv, eps=self.eps, weight=self.norm_weight,
                          gate=proj[:, 2 * self.cq + self.cv:] if self.gate is not None else None, gate_activation=self.gate)
         return linear(out, self.o_weight, out_dtype=self.result_dtype)
 
-    def recur(self, o, proj, state, batch, cols):
+    def recur(self, o, proj, state, batch, cols, prepare=None):
         """o[n] = S^T q over the step's tokens, and the requests' states brought up to date: token by token where every
         request brings few, in runs of 64 tokens on the matrix cores where one brings many."""
         if batch.max_count > self.SCAN_UP_TO and self.head_dim <= ops.DECAY_CHUNKS_MAX_KEY:
+            if prepare is not None:
+                ops.decay_prepare(proj, **prepare, **cols)
             ops.decay_chunks(o, proj, state, batch.state_slots, batch.cu_seqlens, batch.context_lens, self.decay,
                              batch.max_count, **cols)
             return
-        ops.decay_scan(o, proj, state, batch.state_slots, batch.cu_seqlens, batch.context_lens, self.decay, **cols)
+        if prepare is not None and batch.max_count > self.SCAN_UP_TO:  # (keys too wide for the runs: many tokens all the same)
+            ops.decay_prepare(proj, **prepare, **cols)
+            prepare = None
+        ops.decay_scan(o, proj, state, batch.state_slots, batch.cu_seqlens, batch.context_lens, self.decay, prepare=prepare,
+                       **cols)

@@ -90,10 +90,13 @@ class Experts(FeedForward):
         ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize, scores=self.scores,
                        groups=self.groups, keep=self.keep, renorm_eps=self.renorm_eps)
         on_input = self.weight_on == "input"
-        rank, seg, tiles = ops.moe_sort(chosen, self.experts)
         sorted_in = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
         place = torch.empty(pairs, dtype=torch.int32, device=dev)
-        ops.moe_scatter(sorted_in, place, x, chosen, weight if on_input else None, rank, seg)
+        if 0 < pairs <= ops.MOE_FEW_PAIRS:  # (decoding: one launch instead of three)
+            seg, tiles = ops.moe_place_few(sorted_in, place, x, chosen, weight if on_input else None, self.experts)
+        else:
+            rank, seg, tiles = ops.moe_sort(chosen, self.experts)
+            ops.moe_scatter(sorted_in, place, x, chosen, weight if on_input else None, rank, seg)
         act = torch.empty((pairs, self.intermediate), dtype=x.dtype, device=dev)
         ops.grouped_product(act, sorted_in, self.w_gate_up, epilogue="paired", segments=(seg, tiles), limit=self.limit,
                             units=self.intermediate, unit=self.unit)

@@ -72,6 +72,36 @@ def test_activation_rotation_and_key_scale(heads, dk, dv, dims, act):
     assert torch.equal(got[:, :pad], proj[:, :pad].float().double()) and torch.equal(got[:, -pad:], proj[:, -pad:].float().double())
 
 
+@pytest.mark.parametrize("heads,dk,dv,dims,act", [(3, 12, 20, 0, "silu"), (2, 16, 8, 8, None), (1, 72, 80, 72, "silu"),
+                                                  (2, 130, 70, 2, "silu"), (4, 8, 8, 4, None)])
+def test_the_recurrence_prepares_what_it_reads_as_the_kernel_of_its_own_does(heads, dk, dv, dims, act):
+    """Token by token the recurrence may take the projection as it is and do the activation, the rotation and the key's
+    factor on the way in: the same numbers as after the preparing kernel, and the projection is left alone."""
+    from llmserve.ops import library as ops
+
+    counts, lengths = [1, 3, 1, 2], [40, 3, 1501, 9]
+    n, pad = sum(counts), 3
+    proj = dev(torch.cat([rnd(n, pad, seed=6), rnd(n, 2 * heads * dk + heads * dv, seed=7), rnd(n, pad, seed=8)], dim=1))
+    positions = [length - c + i for c, length in zip(counts, lengths) for i in range(c)]
+    freq = None if not dims else dev(torch.tensor([70.0 ** (-2.0 * i / dims) for i in range(dims // 2)], dtype=F64))
+    cols = dict(col_q=pad, col_k=pad + heads * dk, col_v=pad + 2 * heads * dk, heads=heads, dk=dk, dv=dv)
+    prepare = dict(activation=act, freq=freq, rot_dims=dims, positions=ints(positions), key_scale=dk ** -0.5)
+    decay = dev(torch.tensor([0.9 + 0.02 * h for h in range(heads)], dtype=F64))
+    cu = ints([0] + list(torch.tensor(counts).cumsum(0)))
+    state0 = dev(rnd(4, heads, dk, dv, seed=9))
+    results = []
+    for fused in (False, True):
+        p, state = proj.clone(), state0.clone()
+        out = torch.full((n, heads * dv), float("nan"), dtype=torch.float32, device=DEV)
+        if not fused:
+            ops.decay_prepare(p, **prepare, **cols)
+        ops.decay_scan(out, p, state, ints([2, 0, 3, 1]), cu, ints(lengths), decay, prepare=prepare if fused else None, **cols)
+        if fused:
+            assert torch.equal(p, proj)
+        results.append((out, state))
+    assert torch.equal(results[0][0], results[1][0]) and torch.equal(results[0][1], results[1][1])
+
+
 SCAN_CASES = [(3, 12, 20), (2, 16, 8), (1, 72, 80), (2, 130, 70), (1, 32, 64), (5, 8, 200)]
 
 
@@ -359,7 +389,7 @@ def test_softmax_scores_and_the_best_groups(experts, top, groups, keep):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("experts,top,ff,groups,keep,rows", [(6, 2, 24, 3, 2, 150), (3, 1, 40, 1, 1, 1), (8, 8, 4, 2, 2, 37),
-                                                             (12, 4, 64, 4, 3, 300)])
+                                                             (10, 3, 48, 5, 3, 300)])
 def test_experts_against_the_plain_sum(dtype, experts, top, ff, groups, keep, rows):
     import llmserve.parts.model  # noqa: F401  (registers the built-in parts)
     from llmserve.parts.registry import FEED_FORWARDS, BuildContext
