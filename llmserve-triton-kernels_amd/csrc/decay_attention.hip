@@ -73,6 +73,33 @@ struct DecayPrep {
     float key_scale;
 };
 
+// Dimension e of a head's q (or, `key`, k) of the token at row `row`, prepared; `src`: the head's numbers in that row.
+template <bool PREP>
+__device__ __forceinline__ float da_take(const float* __restrict__ src, int e, bool key, const DecayPrep& prep, int row) {
+    float x = src[e];
+    if constexpr (PREP) {
+        if (prep.act == DA_ACT_SILU) x = da_silu(x);
+        if (e < prep.rot_dims) {  // dimension e < half is turned together with dimension e + half
+            const int half = prep.rot_dims / 2;
+            const bool first = e < half;
+            float y = src[first ? e + half : e - half];
+            if (prep.act == DA_ACT_SILU) y = da_silu(y);
+            const float2 sc = rotary_angle((float)prep.positions[row], prep.freq[first ? e : e - half]);
+            const float2 turned = first ? rotate_pair(x, y, sc.y, sc.x) : rotate_pair(y, x, sc.y, sc.x);
+            x = first ? turned.x : turned.y;
+        }
+        if (key) x *= prep.key_scale;
+    }
+    return x;
+}
+
+template <bool PREP>
+__device__ __forceinline__ float da_take_value(float v, const DecayPrep& prep) {
+    if constexpr (PREP)
+        if (prep.act == DA_ACT_SILU) v = da_silu(v);
+    return v;
+}
+
 template <int RPT, bool PREP>
 __global__ __launch_bounds__(DA_THREADS) void decay_scan_kernel(
     float* __restrict__ out, int out_stride, const float* __restrict__ proj, int stride, int col_q, int col_k, int col_v,
@@ -102,27 +129,9 @@ __global__ __launch_bounds__(DA_THREADS) void decay_scan_kernel(
         float* buf = qk[t & 1];
         for (int i = threadIdx.x; i < 2 * dk; i += DA_THREADS) {
             const bool key = i >= dk;
-            const int e = key ? i - dk : i;
-            const float* src = row + (key ? col_k : col_q) + h * dk;
-            float x = src[e];
-            if constexpr (PREP) {
-                if (prep.act == DA_ACT_SILU) x = da_silu(x);
-                if (e < prep.rot_dims) {  // dimension e < half is turned together with dimension e + half
-                    const int half = prep.rot_dims / 2;
-                    const bool first = e < half;
-                    float y = src[first ? e + half : e - half];
-                    if (prep.act == DA_ACT_SILU) y = da_silu(y);
-                    const float2 sc = rotary_angle((float)prep.positions[row0 + t], prep.freq[first ? e : e - half]);
-                    const float2 turned = first ? rotate_pair(x, y, sc.y, sc.x) : rotate_pair(y, x, sc.y, sc.x);
-                    x = first ? turned.x : turned.y;
-                }
-                if (key) x *= prep.key_scale;
-            }
-            buf[i] = x;
+            buf[i] = da_take<PREP>(row + (key ? col_k : col_q) + h * dk, key ? i - dk : i, key, prep, row0 + t);
         }
-        float v = c < dv ? row[col_v + h * dv + c] : 0.f;
-        if constexpr (PREP)
-            if (prep.act == DA_ACT_SILU) v = da_silu(v);
+        const float v = c < dv ? da_take_value<PREP>(row[col_v + h * dv + c], prep) : 0.f;
         __syncthreads();
         // (the sums of the token before, left in the other buffer, are added up behind this barrier)
         if (t > 0 && r == 0 && c < dv) {
@@ -177,11 +186,11 @@ __device__ __forceinline__ int da_run_place(int row0, int b, int j) { return row
 
 // grid: (runs of the longest portion, heads, requests * slabs).  ws[run][h] = sum_t decay^(n - 1 - t) k_t v_t^T over the
 // run's n tokens.
-template <int DKP>
+template <int DKP, bool PREP>
 __global__ __launch_bounds__(DA_THREADS) void decay_chunk_sums_kernel(
     float* __restrict__ ws, const float* __restrict__ proj, int stride, int col_k, int col_v,
     const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens, const float* __restrict__ decay, int heads,
-    int dk, int dv, int slabs) {
+    int dk, int dv, int slabs, const DecayPrep prep) {
     constexpr int LD = DKP + 1, LV = DA_SLAB + 1;
     __shared__ float ks[DA_CHUNK * LD];
     __shared__ float vs[DA_CHUNK * LV];
@@ -195,11 +204,13 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_sums_kernel(
     const float* rows = proj + (size_t)(row0 + j * DA_CHUNK) * stride;
     for (int e = threadIdx.x; e < DA_CHUNK * DKP; e += DA_THREADS) {
         const int t = e / DKP, i = e % DKP;
-        ks[t * LD + i] = (t < n && i < dk) ? rows[(size_t)t * stride + col_k + h * dk + i] * powers[n - 1 - t] : 0.f;
+        ks[t * LD + i] = (t < n && i < dk) ? da_take<PREP>(rows + (size_t)t * stride + col_k + h * dk, i, true, prep,
+                                                           row0 + j * DA_CHUNK + t) * powers[n - 1 - t]
+                                           : 0.f;
     }
     for (int e = threadIdx.x; e < DA_CHUNK * DA_SLAB; e += DA_THREADS) {
         const int t = e / DA_SLAB, c = e % DA_SLAB;
-        vs[t * LV + c] = (t < n && c0 + c < dv) ? rows[(size_t)t * stride + col_v + h * dv + c0 + c] : 0.f;
+        vs[t * LV + c] = (t < n && c0 + c < dv) ? da_take_value<PREP>(rows[(size_t)t * stride + col_v + h * dv + c0 + c], prep) : 0.f;
     }
     __syncthreads();
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, lo = lane % 32, hi = lane / 32;
@@ -249,11 +260,11 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_scan_kernel(
 
 // grid: (runs of the longest portion, heads, requests * slabs).  o_t = decay^(t + 1) S^T q_t + sum_(s <= t) (q_t . k_s)
 // decay^(t - s) v_s over the run's tokens, S being the state before the run (ws[run][h]).
-template <int DKP>
+template <int DKP, bool PREP>
 __global__ __launch_bounds__(DA_THREADS) void decay_chunk_out_kernel(
     float* __restrict__ out, int out_stride, const float* __restrict__ ws, const float* __restrict__ proj, int stride, int col_q,
     int col_k, int col_v, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
-    const float* __restrict__ decay, int heads, int dk, int dv, int slabs) {
+    const float* __restrict__ decay, int heads, int dk, int dv, int slabs, const DecayPrep prep) {
     constexpr int LD = DKP + 1, LV = DA_SLAB + 1, LP = DA_CHUNK + 1;
     constexpr int KS = DA_CHUNK * LD > DKP * LV ? DA_CHUNK * LD : DKP * LV;  // the keys, and after them the state's columns
     extern __shared__ float lds[];
@@ -276,12 +287,13 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_out_kernel(
     for (int e = threadIdx.x; e < DA_CHUNK * DKP; e += DA_THREADS) {
         const int t = e / DKP, i = e % DKP;
         const bool there = t < n && i < dk;
-        qs[t * LD + i] = there ? rows[(size_t)t * stride + col_q + h * dk + i] : 0.f;
-        ks[t * LD + i] = there ? rows[(size_t)t * stride + col_k + h * dk + i] : 0.f;
+        const int row = row0 + j * DA_CHUNK + t;
+        qs[t * LD + i] = there ? da_take<PREP>(rows + (size_t)t * stride + col_q + h * dk, i, false, prep, row) : 0.f;
+        ks[t * LD + i] = there ? da_take<PREP>(rows + (size_t)t * stride + col_k + h * dk, i, true, prep, row) : 0.f;
     }
     for (int e = threadIdx.x; e < DA_CHUNK * DA_SLAB; e += DA_THREADS) {
         const int t = e / DA_SLAB, c = e % DA_SLAB;
-        vs[t * LV + c] = (t < n && c0 + c < dv) ? rows[(size_t)t * stride + col_v + h * dv + c0 + c] : 0.f;
+        vs[t * LV + c] = (t < n && c0 + c < dv) ? da_take_value<PREP>(rows[(size_t)t * stride + col_v + h * dv + c0 + c], prep) : 0.f;
     }
     __syncthreads();
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, lo = lane % 32, hi = lane / 32;
@@ -428,7 +440,8 @@ long long llms_decay_chunks_workspace(int n_tokens, int n_seqs, int heads, int d
 // The same recurrence as llms_decay_scan for portions of many tokens (`max_new`: the most one request brings).
 int llms_decay_chunks(float* out, int out_stride, const float* proj, int stride, int col_q, int col_k, int col_v, float* state,
                       const int* state_slots, const int* cu_seqlens, const int* context_lens, const float* decay, float* ws,
-                      int n_seqs, int max_new, int heads, int dk, int dv, hipStream_t stream) {
+                      int n_seqs, int max_new, int heads, int dk, int dv, int prepare, const int* positions, const float* freq,
+                      int rot_dims, int act, float key_scale, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && dk > 0 && dv > 0, "decay_chunks: sizes must be positive");
     LLMS_REQUIRE(dk <= 128, "decay_chunks: keys of up to 128 numbers");
     LLMS_REQUIRE(ws, "decay_chunks: a workspace");
@@ -436,27 +449,39 @@ int llms_decay_chunks(float* out, int out_stride, const float* proj, int stride,
     LLMS_REQUIRE(heads <= 65535 && (long long)n_seqs * slabs <= 65535, "decay_chunks: up to 65,535 heads, and requests times slabs");
     const dim3 grid(runs, heads, n_seqs * slabs);
     const int dkp = (dk + 31) / 32 * 32;
+    if (prepare) {
+        LLMS_REQUIRE(rot_dims >= 0 && rot_dims <= dk && rot_dims % 2 == 0, "decay_chunks: an even number of turned dimensions, up to dk");
+        LLMS_REQUIRE(rot_dims == 0 || (freq && positions), "decay_chunks: a rotation needs frequencies and positions");
+        LLMS_REQUIRE(act == DA_ACT_NONE || act == DA_ACT_SILU, "decay_chunks: activation 0 (none) or 1 (SiLU)");
+    }
+    const DecayPrep prep = {positions, freq, rot_dims, act, key_scale};
 #define DA_GO(DKP)                                                                                                        \
     do {                                                                                                                  \
-        decay_chunk_sums_kernel<DKP><<<grid, DA_THREADS, 0, stream>>>(ws, proj, stride, col_k, col_v, cu_seqlens,          \
-                                                                      context_lens, decay, heads, dk, dv, slabs);         \
+        if (prepare) DA_GO2(DKP, true);                                                                                   \
+        else DA_GO2(DKP, false);                                                                                          \
+    } while (0)
+#define DA_GO2(DKP, PREP)                                                                                                        \
+    do {                                                                                                                  \
+        decay_chunk_sums_kernel<DKP, PREP><<<grid, DA_THREADS, 0, stream>>>(ws, proj, stride, col_k, col_v, cu_seqlens,    \
+                                                                            context_lens, decay, heads, dk, dv, slabs, prep); \
         decay_chunk_scan_kernel<<<dim3((dk * dv + DA_THREADS - 1) / DA_THREADS, heads, n_seqs), DA_THREADS, 0, stream>>>(   \
             ws, state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv);                                      \
         constexpr int ks = DA_CHUNK * (DKP + 1) > DKP * (DA_SLAB + 1) ? DA_CHUNK * (DKP + 1) : DKP * (DA_SLAB + 1);       \
         const size_t lds = (size_t)(DA_CHUNK * (DKP + 1) + ks + DA_CHUNK * (DA_CHUNK + 1) + DA_CHUNK * (DA_SLAB + 1) +    \
                                     DA_CHUNK + 1) * sizeof(float);                                                        \
         if (lds > 48 * 1024)                                                                                              \
-            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)decay_chunk_out_kernel<DKP>,                                  \
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)decay_chunk_out_kernel<DKP, PREP>,                            \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                    \
-        decay_chunk_out_kernel<DKP><<<grid, DA_THREADS, lds, stream>>>(out, out_stride, ws, proj, stride, col_q, col_k,    \
-                                                                       col_v, cu_seqlens, context_lens, decay, heads, dk, \
-                                                                       dv, slabs);                                        \
+        decay_chunk_out_kernel<DKP, PREP><<<grid, DA_THREADS, lds, stream>>>(out, out_stride, ws, proj, stride, col_q,     \
+                                                                             col_k, col_v, cu_seqlens, context_lens,      \
+                                                                             decay, heads, dk, dv, slabs, prep);          \
     } while (0)
     if (dkp == 32) DA_GO(32);
     else if (dkp == 64) DA_GO(64);
     else if (dkp == 96) DA_GO(96);
     else DA_GO(128);
 #undef DA_GO
+#undef DA_GO2
     LLMS_LAUNCH_CHECK();
 }
 

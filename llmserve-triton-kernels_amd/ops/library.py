@@ -1766,6 +1766,26 @@ def _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk,
     return b
 
 
+def _decay_prepare_args(prepare: dict | None, proj: torch.Tensor, dk: int) -> tuple:
+    """The trailing arguments of the kernels that prepare q, k and v on their way in: (whether, positions, freq,
+    rot_dims, activation, key_scale) from the keyword arguments of `decay_prepare` (None: nothing to prepare)."""
+    if prepare is None:
+        return c_int(0), None, None, c_int(0), c_int(0), c_float(1.0)
+    if prepare.get("activation") not in (None, "none", "silu"):
+        raise ValueError(f"activation {prepare.get('activation')!r}")
+    rot = int(prepare.get("rot_dims") or 0)
+    if rot % 2 or not 0 <= rot <= dk:
+        raise ValueError("rot_dims must be even and at most dk")
+    positions = freq = None
+    if rot:
+        positions, freq = prepare.get("positions"), prepare.get("freq")
+        _f32(freq, "freq", rot // 2)
+        _i32(positions, "positions", proj.shape[0])
+        _dev(proj, freq, positions)
+    return (c_int(1), _ptr(positions), _ptr(freq), c_int(rot), c_int(_ACTIVATIONS[prepare.get("activation")]),
+            c_float(float(prepare.get("key_scale", 1.0))))
+
+
 def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
                cu_seqlens: torch.Tensor, context_lens: torch.Tensor, decay: torch.Tensor, *, col_q: int, col_k: int,
                col_v: int, heads: int, dk: int, dv: int, prepare: dict | None = None) -> torch.Tensor:
@@ -1778,17 +1798,7 @@ def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state
     `decay_prepare` would do to q, k and v is done on their way in, with the same arithmetic (proj is not written)."""
     dev = _dev(out, proj, state, state_slots, cu_seqlens, context_lens, decay)
     _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
-    prep = prepare or {}
-    p_positions, p_freq, p_rot = prep.get("positions"), prep.get("freq"), int(prep.get("rot_dims") or 0)
-    if prepare is not None:
-        if prep.get("activation") not in (None, "none", "silu"):
-            raise ValueError(f"activation {prep.get('activation')!r}")
-        if p_rot % 2 or not 0 <= p_rot <= dk:
-            raise ValueError("rot_dims must be even and at most dk")
-        if p_rot:
-            _f32(p_freq, "freq", p_rot // 2)
-            _i32(p_positions, "positions", proj.shape[0])
-            _dev(out, p_freq, p_positions)
+    prep_args = _decay_prepare_args(prepare, proj, dk)
     if out.dtype != torch.float32 or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (proj.shape[0], heads * dv):
         raise ValueError(f"out must be float32 [{proj.shape[0]}, {heads * dv}] with unit inner stride")
     if dk > DECAY_MAX_KEY:
@@ -1799,22 +1809,21 @@ def decay_scan(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state
     _check(load("decay_attention").llms_decay_scan(
         _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
         _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), c_int(b), c_int(heads), c_int(dk),
-        c_int(dv), c_int(0 if prepare is None else 1), _ptr(p_positions if p_rot else None), _ptr(p_freq if p_rot else None),
-        c_int(p_rot), c_int(_ACTIVATIONS[prep.get("activation")] if prepare is not None else 0),
-        c_float(float(prep.get("key_scale", 1.0))), _stream(dev)), "decay_scan")
+        c_int(dv), *prep_args, _stream(dev)), "decay_scan")
     return out
 
 
 DECAY_CHUNKS_MAX_KEY = 128  # numbers of a key that `decay_chunks` takes
+DECAY_CHUNKS_SLAB = 64  # columns of v that one of its workgroups takes
 
 
 def decay_chunks(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
                  cu_seqlens: torch.Tensor, context_lens: torch.Tensor, decay: torch.Tensor, max_new: int, *, col_q: int,
-                 col_k: int, col_v: int, heads: int, dk: int, dv: int) -> torch.Tensor:
+                 col_k: int, col_v: int, heads: int, dk: int, dv: int, prepare: dict | None = None) -> torch.Tensor:
     """What `decay_scan` computes, for portions of many tokens (`max_new`: the most one request brings): runs of 64
     tokens gather their own sums of k v^T, a scan over the runs gives the state before each and the request's last
     state, and every run adds what its tokens see of each other to what they see of that state; all products on the
-    32-bit matrix instruction.  Same arguments, and the same result up to the order of the sums."""
+    32-bit matrix instruction.  Same arguments (also `prepare`), and the same result up to the order of the sums."""
     dev = _dev(out, proj, state, state_slots, cu_seqlens, context_lens, decay)
     _decay_proj(proj, col_q, col_k, col_v, heads, dk, dv)
     if out.dtype != torch.float32 or out.dim() != 2 or out.stride(1) != 1 or tuple(out.shape) != (proj.shape[0], heads * dv):
@@ -1824,6 +1833,7 @@ def decay_chunks(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, sta
     b = _decay_state(state, state_slots, cu_seqlens, context_lens, decay, heads, dk, dv)
     if b <= 0 or proj.shape[0] == 0 or max_new <= 0:
         return out
+    prep_args = _decay_prepare_args(prepare, proj, dk)
     lib = load("decay_attention")
     lib.llms_decay_chunks_workspace.restype = ctypes.c_longlong
     floats = int(lib.llms_decay_chunks_workspace(c_int(proj.shape[0]), c_int(b), c_int(heads), c_int(dk), c_int(dv)))
@@ -1831,7 +1841,7 @@ def decay_chunks(out: torch.Tensor, proj: torch.Tensor, state: torch.Tensor, sta
     _check(lib.llms_decay_chunks(
         _ptr(out), c_int(out.stride(0)), _ptr(proj), c_int(proj.stride(0)), c_int(col_q), c_int(col_k), c_int(col_v),
         _ptr(state), _ptr(state_slots), _ptr(cu_seqlens), _ptr(context_lens), _ptr(decay), _ptr(ws), c_int(b), c_int(max_new),
-        c_int(heads), c_int(dk), c_int(dv), _stream(dev)), "decay_chunks")
+        c_int(heads), c_int(dk), c_int(dv), *prep_args, _stream(dev)), "decay_chunks")
     return out
 
 

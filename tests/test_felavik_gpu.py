@@ -74,12 +74,16 @@ def test_activation_rotation_and_key_scale(heads, dk, dv, dims, act):
 
 @pytest.mark.parametrize("heads,dk,dv,dims,act", [(3, 12, 20, 0, "silu"), (2, 16, 8, 8, None), (1, 72, 80, 72, "silu"),
                                                   (2, 130, 70, 2, "silu"), (4, 8, 8, 4, None)])
-def test_the_recurrence_prepares_what_it_reads_as_the_kernel_of_its_own_does(heads, dk, dv, dims, act):
-    """Token by token the recurrence may take the projection as it is and do the activation, the rotation and the key's
-    factor on the way in: the same numbers as after the preparing kernel, and the projection is left alone."""
+@pytest.mark.parametrize("kernel", ["scan", "chunks"])
+def test_the_recurrence_prepares_what_it_reads_as_the_kernel_of_its_own_does(heads, dk, dv, dims, act, kernel):
+    """The recurrence may take the projection as it is and do the activation, the rotation and the key's factor on the
+    way in: the same numbers as after the preparing kernel, and the projection is left alone."""
     from llmserve.ops import library as ops
 
-    counts, lengths = [1, 3, 1, 2], [40, 3, 1501, 9]
+    chunks = kernel == "chunks"
+    if chunks and dk > ops.DECAY_CHUNKS_MAX_KEY:
+        pytest.skip("keys wider than the kernel of runs takes")
+    counts, lengths = ([70, 3, 1, 130], [70, 40, 1501, 139]) if chunks else ([1, 3, 1, 2], [40, 3, 1501, 9])
     n, pad = sum(counts), 3
     proj = dev(torch.cat([rnd(n, pad, seed=6), rnd(n, 2 * heads * dk + heads * dv, seed=7), rnd(n, pad, seed=8)], dim=1))
     positions = [length - c + i for c, length in zip(counts, lengths) for i in range(c)]
@@ -95,7 +99,11 @@ def test_the_recurrence_prepares_what_it_reads_as_the_kernel_of_its_own_does(hea
         out = torch.full((n, heads * dv), float("nan"), dtype=torch.float32, device=DEV)
         if not fused:
             ops.decay_prepare(p, **prepare, **cols)
-        ops.decay_scan(out, p, state, ints([2, 0, 3, 1]), cu, ints(lengths), decay, prepare=prepare if fused else None, **cols)
+        args = (out, p, state, ints([2, 0, 3, 1]), cu, ints(lengths), decay)
+        if chunks:
+            ops.decay_chunks(*args, max(counts), prepare=prepare if fused else None, **cols)
+        else:
+            ops.decay_scan(*args, prepare=prepare if fused else None, **cols)
         if fused:
             assert torch.equal(p, proj)
         results.append((out, state))
