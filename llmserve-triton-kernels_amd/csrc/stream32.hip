@@ -358,6 +358,63 @@ __global__ __launch_bounds__(S32_THREADS) void streams_norm_vec_kernel(
     }
 }
 
+// One stream (S = 1) with rows of 256 V numbers, V up to 16: a wave takes a row and keeps it in registers (V float4 a
+// lane), so the row costs one wait for memory, no LDS and no barrier; a workgroup is 4 rows.  The same arithmetic per
+// element as above (new = mix x + write y, u = read new); the sums of a row are formed lane by lane and then across
+// the wave, in an order that depends on the row's length alone.
+template <typename T, int V>
+__global__ __launch_bounds__(S32_THREADS) void streams_norm_wave_kernel(
+    T* __restrict__ out, float* x_dst, const float* x_src, const float* __restrict__ y, const float* __restrict__ mix,
+    const float* __restrict__ wout, const float* __restrict__ read, const float* __restrict__ weight,
+    const int* __restrict__ rows, int n_out, int hidden, float eps, int store, int center) {
+    const int lane = threadIdx.x % LLMS_WAVE, r = blockIdx.x * (S32_THREADS / LLMS_WAVE) + threadIdx.x / LLMS_WAVE;
+    if (r >= n_out) return;
+    const int n = rows ? rows[r] : r;
+    const float4* src = reinterpret_cast<const float4*>(x_src + (size_t)n * hidden);
+    const float4* ys = y ? reinterpret_cast<const float4*>(y + (size_t)n * hidden) : nullptr;
+    float4 u[V], yv[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        u[v] = src[v * LLMS_WAVE + lane];
+        yv[v] = ys ? ys[v * LLMS_WAVE + lane] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    const float cm = mix ? mix[0] : 1.f, co = wout ? wout[0] : 1.f, cr = read ? read[0] : 1.f;
+    float total = 0.f;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        float4 w4 = u[v];
+        if (ys) {
+            w4.x = fmaf(co, yv[v].x, cm * w4.x), w4.y = fmaf(co, yv[v].y, cm * w4.y);
+            w4.z = fmaf(co, yv[v].z, cm * w4.z), w4.w = fmaf(co, yv[v].w, cm * w4.w);
+        }
+        if (store) reinterpret_cast<float4*>(x_dst + (size_t)n * hidden)[v * LLMS_WAVE + lane] = w4;
+        u[v] = make_float4(cr * w4.x, cr * w4.y, cr * w4.z, cr * w4.w);
+        total += (u[v].x + u[v].y) + (u[v].z + u[v].w);
+    }
+    if (!out) return;
+    const float mean = center ? wave_sum(total) / (float)hidden : 0.f;
+    float dev2 = 0.f;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const float a = u[v].x - mean, b = u[v].y - mean, c = u[v].z - mean, d = u[v].w - mean;
+        dev2 += (a * a + b * b) + (c * c + d * d);
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(dev2) / (float)hidden + eps);
+    T* orow = out + (size_t)r * hidden;
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        const int c4 = v * LLMS_WAVE + lane;
+        const float4 w4 = reinterpret_cast<const float4*>(weight)[c4];
+        const float a = (u[v].x - mean) * inv * w4.x, b = (u[v].y - mean) * inv * w4.y;
+        const float c = (u[v].z - mean) * inv * w4.z, d = (u[v].w - mean) * inv * w4.w;
+        if constexpr (sizeof(T) == 2) {
+            *reinterpret_cast<uint2*>(orow + 4 * c4) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(c, d));
+        } else {
+            *reinterpret_cast<float4*>(orow + 4 * c4) = make_float4(a, b, c, d);
+        }
+    }
+}
+
 // x <- cap * tanh(x / cap), in place on 32-bit numbers (logits)
 __global__ void softcap_kernel(float* __restrict__ x, size_t total, float cap) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -471,6 +528,28 @@ int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, in
     const size_t lds = (size_t)hidden * sizeof(float);
     auto aligned = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
     const bool vec = hidden % 4 == 0 && aligned(x_dst) && aligned(x_src) && aligned(y) && aligned(weight) && aligned(out);
+    // one stream with rows of 256, 512, 1,024, 2,048 or 4,096 numbers: a wave a row, the row in registers
+    const int per_lane = hidden % (4 * LLMS_WAVE) == 0 ? hidden / (4 * LLMS_WAVE) : 0;
+    if (vec && streams == 1 && (per_lane == 1 || per_lane == 2 || per_lane == 4 || per_lane == 8 || per_lane == 16)) {
+        const int per_wg = S32_THREADS / LLMS_WAVE;
+        const dim3 grid((n_out + per_wg - 1) / per_wg);
+#define WAVE_GO(V)                                                                                                          \
+    do {                                                                                                                    \
+        if (dtype == 0)                                                                                                     \
+            streams_norm_wave_kernel<float, V><<<grid, S32_THREADS, 0, stream>>>((float*)out, x_dst, x_src, y, mix, wout, read, \
+                                                                                 weight, rows, n_out, hidden, eps, store, center); \
+        else                                                                                                                \
+            streams_norm_wave_kernel<bf16, V><<<grid, S32_THREADS, 0, stream>>>((bf16*)out, x_dst, x_src, y, mix, wout, read, \
+                                                                                weight, rows, n_out, hidden, eps, store, center); \
+    } while (0)
+        if (per_lane == 1) WAVE_GO(1);
+        else if (per_lane == 2) WAVE_GO(2);
+        else if (per_lane == 4) WAVE_GO(4);
+        else if (per_lane == 8) WAVE_GO(8);
+        else WAVE_GO(16);
+#undef WAVE_GO
+        LLMS_LAUNCH_CHECK();
+    }
 #define STREAMS_GO(KERNEL, T)                                                                                               \
     do {                                                                                                                    \
         if (lds > 32 * 1024)                                                                                                \

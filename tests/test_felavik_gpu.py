@@ -423,13 +423,29 @@ def test_the_soft_cap_the_weighted_sum_and_the_norm_without_a_mean():
     a, b = rnd(7, 50, seed=2), rnd(7, 50, seed=3)
     da = dev(a)
     close(ops.weighted_sum(da, da, dev(b), 0.8, -1.1), 0.8 * a - 1.1 * b, torch.float32, "weighted sum in place")
-    for hidden in (100, 98, 2048):
-        x, y, w = rnd(4, hidden, seed=4, scale=3.0) + 0.7, rnd(4, hidden, seed=5), rnd(hidden, seed=6) + 1
-        stream = dev(x).unsqueeze(1).contiguous()
-        out = torch.empty((4, hidden), dtype=torch.float32, device=DEV)
-        ops.streams_norm(out, stream, dev(w), 1e-5, y=dev(y), center=False)
-        close(out, pf.rms_norm(x + y, w, 1e-5), torch.float32, "RMS norm of the closed sum")
-        close(stream[:, 0], x + y, torch.float32, "the sum stored")
+    for hidden in (100, 98, 256, 512, 1024, 2048, 4096, 768, 8192):  # (a wave a row at 256 .. 4,096; a workgroup a row else)
+        n = 7
+        x, y, w = rnd(n, hidden, seed=4, scale=3.0) + 0.7, rnd(n, hidden, seed=5), rnd(hidden, seed=6) + 1
+        for dtype in DTYPES:
+            stream = dev(x).unsqueeze(1).contiguous()
+            out = torch.full((n, hidden), float("nan"), dtype=dtype, device=DEV)
+            ops.streams_norm(out, stream, dev(w), 1e-5, y=dev(y), center=False)
+            close(out, pf.rms_norm(x + y, w, 1e-5), dtype, f"RMS norm of the closed sum, {hidden}")
+            close(stream[:, 0], x + y, torch.float32, "the sum stored")
+            # the first read of a layer: the rows as they are; picked rows: nothing stored
+            again = torch.full((n, hidden), float("nan"), dtype=dtype, device=DEV)
+            ops.streams_norm(again, stream, dev(w), 1e-5, center=False)
+            assert torch.equal(again, out)
+            picked = torch.full((3, hidden), float("nan"), dtype=dtype, device=DEV)
+            before = stream.clone()
+            ops.streams_norm(picked, stream, dev(w), 1e-5, y=dev(y), rows=ints([6, 0, 3]), center=False)
+            close(picked, pf.rms_norm(x + 2 * y, w, 1e-5)[[6, 0, 3]], dtype, f"picked rows, {hidden}")
+            assert torch.equal(stream, before)
+            centered = torch.empty((n, hidden), dtype=torch.float32, device=DEV)
+            ops.streams_norm(centered, stream, dev(w), 1e-5, center=True)
+            z = x + y
+            want = (z - z.mean(-1, keepdim=True)) / torch.sqrt(z.var(-1, unbiased=False, keepdim=True) + 1e-5) * w
+            close(centered, want, torch.float32, f"with the mean taken off, {hidden}")
 
 
 # ------------------------------------------------------------------------------ whole models
