@@ -128,9 +128,8 @@ static int launch_fma(int epilogue, dim3 grid, hipStream_t stream, void* out, lo
 }
 
 // ------------------------------------------------------------------------------ bfloat16 on the matrix cores
-// 128 x 128 tiles, 64 of K at a time, through double-buffered LDS (72 KB: two workgroups a compute unit; a tile of
-// K in flight is 32 KB a workgroup, which is what lets few rows stream the weights near the memory's rate), 4 waves of
-// 64 x 64, v_mfma_f32_32x32x16_bf16: lane l holds
+// 128 x 128 tiles, 64 of K at a time, through double-buffered LDS (72 KB: two workgroups a compute unit) with two more
+// tiles of K in flight in registers, 4 waves of 64 x 64, v_mfma_f32_32x32x16_bf16: lane l holds
 // A[i = l%32][k = 8*(l/32) .. +7] and B[k = same][j = l%32]; result D[i = 8*(r/4) + 4*(l/32) + r%4][j = l%32].
 // Here i = row m and j = weight row n, so a wave's two column blocks of 32 are the a and b rows of the same 32 units
 // of a paired weight (columns 0..31 and 32..63 of its 64), both in the same lane.
@@ -181,54 +180,61 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    // staging: 1,024 pieces of 8 elements per operand tile, four per thread
-    gg_u32x4 ra[GM_PIECES], rb[GM_PIECES];
+    // staging: 1,024 pieces of 8 elements per operand tile, four per thread.  Two tiles of K are in flight in two sets of
+    // registers (set kt % 2 holds tile kt) beside the tile in LDS that is being multiplied: 64 KB a workgroup, which is what
+    // lets few rows stream the weights near the memory's rate, and many rows hide a trip to memory behind two tiles' products.
+    // A piece beyond the rows, the weight or K is not asked for and counts as zeros, so tiles past the last are fetched too.
+    gg_u32x4 ra0[GM_PIECES], rb0[GM_PIECES], ra1[GM_PIECES], rb1[GM_PIECES];
     const int crow0 = tid / 8, ckc = (tid % 8) * 8;
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int c = 0; c < GM_PIECES; ++c) {
-            const int k = k0 + ckc;
-            const int am = row0 + crow0 + 32 * c, wr = n0 + crow0 + 32 * c;
-            ra[c] = (am < row_end && k < K) ? *reinterpret_cast<const gg_u32x4*>(xg + (size_t)am * x_ld + k) : zero;
-            rb[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * w_ld + k) : zero;
-        }
-    };
-    auto stage = [&](int buf) {
-#pragma unroll
-        for (int c = 0; c < GM_PIECES; ++c) {
-            *reinterpret_cast<gg_u32x4*>(&As[buf][(crow0 + 32 * c) * GM_LD + ckc]) = ra[c];
-            *reinterpret_cast<gg_u32x4*>(&Bs[buf][(crow0 + 32 * c) * GM_LD + ckc]) = rb[c];
-        }
-    };
     // (with segments the third grid dimension may share K out: part p takes k_part numbers from p * k_part on and
     // leaves its sums in an array of its own, for the caller to add up)
     const int k_begin = seg ? blockIdx.z * k_part : 0;
     const int k_end = seg ? min(K, k_begin + k_part) : K;
     const int ktiles = (k_end - k_begin + GM_BK - 1) / GM_BK;
     K = k_end;
-    fetch(k_begin);
-    stage(0);
+#define GM_FETCH(RA, RB, K0)                                                                                               \
+    _Pragma("unroll") for (int c = 0; c < GM_PIECES; ++c) {                                                                \
+        const int k = (K0) + ckc;                                                                                          \
+        const int am = row0 + crow0 + 32 * c, wr = n0 + crow0 + 32 * c;                                                    \
+        RA[c] = (am < row_end && k < K) ? *reinterpret_cast<const gg_u32x4*>(xg + (size_t)am * x_ld + k) : zero;           \
+        RB[c] = (wr < N && k < K) ? *reinterpret_cast<const gg_u32x4*>(wg + (size_t)wr * w_ld + k) : zero;                 \
+    }
+#define GM_STAGE(BUF, RA, RB)                                                                                              \
+    _Pragma("unroll") for (int c = 0; c < GM_PIECES; ++c) {                                                                \
+        *reinterpret_cast<gg_u32x4*>(&As[BUF][(crow0 + 32 * c) * GM_LD + ckc]) = RA[c];                                    \
+        *reinterpret_cast<gg_u32x4*>(&Bs[BUF][(crow0 + 32 * c) * GM_LD + ckc]) = RB[c];                                    \
+    }
+#define GM_MULTIPLY(BUF)                                                                                                   \
+    _Pragma("unroll") for (int s = 0; s < GM_BK / 16; ++s) {                                                               \
+        gg_bf16x8 af[2], bfr[2];                                                                                           \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i) {                                                                    \
+            af[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&As[BUF][(wm + i * 32 + l32) * GM_LD + s * 16 + hi * 8])); \
+            bfr[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&Bs[BUF][(wn + i * 32 + l32) * GM_LD + s * 16 + hi * 8])); \
+        }                                                                                                                  \
+        _Pragma("unroll") for (int i = 0; i < 2; ++i)                                                                      \
+            _Pragma("unroll") for (int j = 0; j < 2; ++j)                                                                  \
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);                    \
+    }
+    GM_FETCH(ra0, rb0, k_begin);
+    GM_FETCH(ra1, rb1, k_begin + GM_BK);
+    GM_STAGE(0, ra0, rb0);
     __syncthreads();
-    for (int kt = 0; kt < ktiles; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < ktiles) fetch(k_begin + (kt + 1) * GM_BK);
-#pragma unroll
-        for (int s = 0; s < GM_BK / 16; ++s) {
-            gg_bf16x8 af[2], bfr[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                af[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&As[buf][(wm + i * 32 + l32) * GM_LD + s * 16 + hi * 8]));
-                bfr[i] = __builtin_bit_cast(gg_bf16x8, *reinterpret_cast<const gg_u32x4*>(&Bs[buf][(wn + i * 32 + l32) * GM_LD + s * 16 + hi * 8]));
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < ktiles) stage(buf ^ 1);
+    for (int kt = 0; kt < ktiles; kt += 2) {
+        // LDS buffer 0 holds tile kt, set 1 tile kt + 1; set 0 is free for tile kt + 2
+        GM_FETCH(ra0, rb0, k_begin + (kt + 2) * GM_BK);
+        GM_MULTIPLY(0);
+        GM_STAGE(1, ra1, rb1);
+        __syncthreads();
+        if (kt + 1 >= ktiles) break;
+        // LDS buffer 1 holds tile kt + 1, set 0 tile kt + 2; set 1 is free for tile kt + 3
+        GM_FETCH(ra1, rb1, k_begin + (kt + 3) * GM_BK);
+        GM_MULTIPLY(1);
+        GM_STAGE(0, ra0, rb0);
         __syncthreads();
     }
+#undef GM_FETCH
+#undef GM_STAGE
+#undef GM_MULTIPLY
     TOut* og = out + (seg ? (size_t)blockIdx.z * part_stride : (size_t)g * out_gs);
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
