@@ -248,12 +248,19 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_scan_kernel(
     float s = length > count ? *st : 0.f;  // (a portion from position 0 starts from zero)
     float* at = ws + ((size_t)da_run_place(row0, b, 0) * heads + h) * dk * dv + e;
     const size_t step = (size_t)heads * dk * dv;
-    float sum = *at;
-    for (int j = 0; j < runs; ++j) {
-        const float next = j + 1 < runs ? at[step] : 0.f;  // (asked for before this run's is overwritten and used)
-        *at = s;
-        s = fmaf(j + 1 < runs ? (float)full : (float)rest, s, sum);
-        sum = next, at += step;
+    for (int j0 = 0; j0 < runs; j0 += 8) {  // 8 runs' sums are asked for together, then replaced one after the other
+        float sums[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sums[u] = j0 + u < runs ? at[(size_t)u * step] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int j = j0 + u;
+            if (j < runs) {
+                at[(size_t)u * step] = s;
+                s = fmaf(j + 1 < runs ? (float)full : (float)rest, s, sums[u]);
+            }
+        }
+        at += 8 * step;
     }
     *st = s;
 }
@@ -295,6 +302,15 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_out_kernel(
         const int t = e / DA_SLAB, c = e % DA_SLAB;
         vs[t * LV + c] = (t < n && c0 + c < dv) ? da_take_value<PREP>(rows[(size_t)t * stride + col_v + h * dv + c0 + c], prep) : 0.f;
     }
+    // the state before the run is asked for now and put into LDS (in the keys' place) once the scores are done with the keys
+    constexpr int S_EACH = DKP * DA_SLAB / DA_THREADS;
+    float s_before[S_EACH];
+    const float* before = ws + ((size_t)da_run_place(row0, b, j) * heads + h) * dk * dv;
+#pragma unroll
+    for (int u = 0; u < S_EACH; ++u) {
+        const int e = threadIdx.x + u * DA_THREADS, i = e / DA_SLAB, c = e % DA_SLAB;
+        s_before[u] = (i < dk && c0 + c < dv) ? before[(size_t)i * dv + c0 + c] : 0.f;
+    }
     __syncthreads();
     const int wave = threadIdx.x / LLMS_WAVE, lane = threadIdx.x % LLMS_WAVE, lo = lane % 32, hi = lane / 32;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -315,10 +331,10 @@ __global__ __launch_bounds__(DA_THREADS) void decay_chunk_out_kernel(
     }
     __syncthreads();  // (the keys are done with)
     float* ss = ks;
-    const float* before = ws + ((size_t)da_run_place(row0, b, j) * heads + h) * dk * dv;
-    for (int e = threadIdx.x; e < DKP * DA_SLAB; e += DA_THREADS) {
-        const int i = e / DA_SLAB, c = e % DA_SLAB;
-        ss[i * LV + c] = (i < dk && c0 + c < dv) ? before[(size_t)i * dv + c0 + c] : 0.f;
+#pragma unroll
+    for (int u = 0; u < S_EACH; ++u) {
+        const int e = threadIdx.x + u * DA_THREADS;
+        ss[(e / DA_SLAB) * LV + e % DA_SLAB] = s_before[u];
     }
     __syncthreads();
     const int tr = (wave % 2) * 32, tc = (wave / 2) * 32;
