@@ -399,6 +399,46 @@ __global__ __launch_bounds__(DA_THREADS) void decay_finish_kernel(
     }
 }
 
+// The same for rows of heads * dv = 1,024 E numbers, E up to 8, in 16-byte pieces: a thread keeps its E pieces of o, of the
+// gate's products and of the weight in registers, all asked for before anything is waited for, so a token costs one trip
+// to memory (decoding is a chain of such trips).  The norm over all heads only (a head's own norm needs the row in LDS).
+template <typename T, int E>
+__global__ __launch_bounds__(DA_THREADS) void decay_finish_joint_kernel(
+    T* __restrict__ out, int out_stride, const float* __restrict__ o, int o_stride, const float* __restrict__ gate,
+    int gate_stride, const float* __restrict__ weight, int width, int gate_act, float eps) {
+    __shared__ float red[16];
+    const int n = blockIdx.x;
+    float4 x[E], z[E], w[E];
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < E; ++u) {
+        const int c = 4 * (u * DA_THREADS + threadIdx.x);
+        x[u] = *reinterpret_cast<const float4*>(o + (size_t)n * o_stride + c);
+        w[u] = *reinterpret_cast<const float4*>(weight + c);
+        z[u] = gate_act != DA_ACT_NONE ? *reinterpret_cast<const float4*>(gate + (size_t)n * gate_stride + c)
+                                       : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < E; ++u) ss += (x[u].x * x[u].x + x[u].y * x[u].y) + (x[u].z * x[u].z + x[u].w * x[u].w);
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+    auto gated = [&](float v, float g) {
+        if (gate_act == DA_ACT_NONE) return v;
+        return v * (gate_act == DA_ACT_SILU ? da_silu(g) : 1.f / (1.f + expf(-g)));
+    };
+#pragma unroll
+    for (int u = 0; u < E; ++u) {
+        const int c = 4 * (u * DA_THREADS + threadIdx.x);
+        const float a = gated(x[u].x * inv * w[u].x, z[u].x), b = gated(x[u].y * inv * w[u].y, z[u].y);
+        const float cc = gated(x[u].z * inv * w[u].z, z[u].z), d = gated(x[u].w * inv * w[u].w, z[u].w);
+        T* at = out + (size_t)n * out_stride + c;
+        if constexpr (sizeof(T) == 2) {
+            *reinterpret_cast<uint2*>(at) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
+        } else {
+            *reinterpret_cast<float4*>(at) = make_float4(a, b, cc, d);
+        }
+    }
+}
+
 extern "C" {
 
 int llms_decay_prepare(float* proj, int stride, int col_q, int col_k, int col_v, const int* positions, const float* freq,
@@ -510,6 +550,28 @@ int llms_decay_finish(int dtype, void* out, int out_stride, const float* o, int 
     LLMS_REQUIRE(gate_act >= 0 && gate_act <= 2, "decay_finish: gate 0 (none), 1 (SiLU) or 2 (sigmoid)");
     const size_t lds = (size_t)heads * dv * sizeof(float);
     LLMS_REQUIRE(lds <= 128 * 1024, "decay_finish: heads times value size up to 32,768");
+    const int width = heads * dv, each = width % (4 * DA_THREADS) == 0 ? width / (4 * DA_THREADS) : 0;
+    auto aligned = [](const void* p, int stride) { return ((uintptr_t)p % 16) == 0 && stride % 4 == 0; };
+    if (joint && (each == 1 || each == 2 || each == 4 || each == 8) && aligned(o, o_stride) && aligned(weight, 0) &&
+        (gate_act == DA_ACT_NONE || aligned(gate, gate_stride)) && aligned(out, dtype == 0 ? out_stride : out_stride / 2) &&
+        (dtype == 0 || out_stride % 4 == 0)) {
+#define DA_JOINT(T, E)                                                                                                    \
+    decay_finish_joint_kernel<T, E><<<n_tokens, DA_THREADS, 0, stream>>>((T*)out, out_stride, o, o_stride, gate, gate_stride, \
+                                                                         weight, width, gate_act, eps)
+#define DA_JOINT_T(T)                                                                                                     \
+    do {                                                                                                                  \
+        if (each == 1) DA_JOINT(T, 1);                                                                                    \
+        else if (each == 2) DA_JOINT(T, 2);                                                                               \
+        else if (each == 4) DA_JOINT(T, 4);                                                                               \
+        else DA_JOINT(T, 8);                                                                                              \
+    } while (0)
+        if (dtype == 0) DA_JOINT_T(float);
+        else if (dtype == 1) DA_JOINT_T(bf16);
+        else LLMS_REQUIRE(false, "decay_finish: dtype must be 0 (float32) or 1 (bfloat16)");
+#undef DA_JOINT_T
+#undef DA_JOINT
+        LLMS_LAUNCH_CHECK();
+    }
 #define DA_GO(T)                                                                                                          \
     do {                                                                                                                  \
         if (lds > 32 * 1024)                                                                                              \

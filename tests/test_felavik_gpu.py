@@ -203,19 +203,24 @@ def test_a_key_far_back_is_still_in_the_state_after_long_decoding():
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,dv,joint,gate", [(3, 20, True, "sigmoid"), (2, 8, False, "silu"), (1, 80, False, None),
-                                                 (300, 4, False, "silu"), (2, 2048, True, "sigmoid")])
+                                                 (300, 4, False, "silu"), (2, 2048, True, "sigmoid"),
+                                                 (4, 256, True, "sigmoid"), (16, 128, True, "silu"), (8, 1024, True, None),
+                                                 (4, 1024, True, "sigmoid"), (4, 256, False, "silu")])
 def test_head_norms_and_gates(dtype, heads, dv, joint, gate):
+    """(Rows of 1,024, 2,048, 4,096 or 8,192 numbers whose gate starts at a multiple of 16 bytes are kept in registers
+    where all heads are normed together; the others go through LDS.)"""
     from llmserve.ops import library as ops
 
     n, eps, width = 6, 1e-3, heads * dv
-    o, z, w = rnd(n, heads, dv, seed=1, scale=4.0), rnd(n, width + 3, seed=2), rnd(width, seed=3) + 1
+    pad = 3 if heads == 2 else 4
+    o, z, w = rnd(n, heads, dv, seed=1, scale=4.0), rnd(n, width + pad, seed=2), rnd(width, seed=3) + 1
     o[2] *= 1e-3  # (eps matters for a small row)
-    out = torch.empty((n, width), dtype=dtype, device=DEV)
+    out = torch.full((n, width), float("nan"), dtype=dtype, device=DEV)
     ops.decay_finish(out, dev(o.reshape(n, width)), heads=heads, dv=dv, eps=eps, weight=dev(w) if joint else None,
-                     gate=dev(z)[:, 3:] if gate else None, gate_activation=gate)
+                     gate=dev(z)[:, pad:] if gate else None, gate_activation=gate)
     want = pf.rms_norm(o.reshape(n, width), w, eps) if joint else pf.rms_unit(o, eps).reshape(n, width)
     if gate:
-        want = want * (pf.silu(z[:, 3:]) if gate == "silu" else torch.sigmoid(z[:, 3:]))
+        want = want * (pf.silu(z[:, pad:]) if gate == "silu" else torch.sigmoid(z[:, pad:]))
     close(out, want, dtype, "normed and gated heads")
 
 
