@@ -9,7 +9,9 @@
 //                 token, conv_store writes the ring itself).
 //   norm_store    the same without a convolution, for queries and keys that are normed head by head: every head of q
 //                 and of k is divided by its root mean square over its dk numbers (eps inside the root) and multiplied by a
-//                 weight that all heads share; q is then multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) at
+//                 weight that all heads share (`unit_norm`: no weight); with `freq` the first rot_dims numbers of every
+//                 head of q and k are turned by the token's position first (dimension i together with dimension
+//                 i + rot_dims / 2, angle position * freq[i]); q is then multiplied by 1 + coef * ln(floor((p + 1) / every) + 1) at
 //                 position p (every 0: no factor); all in 32-bit, rounded once, into the query rows and the cache slots.
 //   attend        one workgroup per new token, all heads.  Score heads s = h * maps + m (maps = 2: two score maps
 //                 per query head over the same values); s reads key head (h / (H / G)) * maps + m, values come from
@@ -17,7 +19,7 @@
 //                     j >= chunk_start(i)  and  (i - j < window  or  j < keep_first)
 //                 (window 0: no window; chunk 0: no chunks).  score = q . k * scale - slope_h * (i - j) + dist_bias[h, min(i - j,
 //                 dist_reach)] (a table per head over the distance, which stays at its last entry beyond dist_reach); softmax over the
-//                 visible keys in 32-bit, normalised before anything else happens to it; optionally the heads' weights
+//                 visible keys in 32-bit, normalised before anything else happens to it; with `sink` the denominator holds one more term exp(0); optionally the heads' weights
 //                 are mixed, w_h = sum_g talk[h, g] w_g; then the values.  maps = 2 ends with o = a_1 - lambda a_2;
 //                 head_norm divides a head's result by its root mean square (eps inside the root) and multiplies
 //                 by out_scale.  With gate products z (32-bit) the result is multiplied by sigmoid(z[n, h * dv + d]).
@@ -102,13 +104,23 @@ __global__ __launch_bounds__(AC_THREADS) void conv_state_kernel(
         ring[(size_t)(pos % (taps - 1)) * channels + c] = proj[(size_t)(first_row + pos - first_pos) * proj_stride + c];
 }
 
+// element d of a head after the rotation of its first rot_dims numbers (pairs i, i + rot_dims / 2)
+__device__ __forceinline__ float turned_element(const float* __restrict__ src, int d, int rot_dims, float position,
+                                                const float* __restrict__ freq) {
+    if (d >= rot_dims) return src[d];
+    const int h = rot_dims >> 1, i = d < h ? d : d - h;
+    const float2 sc = rotary_angle(position, freq[i]);  // (sine, cosine)
+    const float2 turned = rotate_pair(src[i], src[i + h], sc.y, sc.x);
+    return d < h ? turned.x : turned.y;
+}
+
 // grid: (tokens, query heads + key heads + value heads); one wave per head
 template <typename T>
 __global__ __launch_bounds__(LLMS_WAVE) void norm_store_kernel(
     T* __restrict__ q_out, int q_stride, const float* __restrict__ proj, int proj_stride, const float* __restrict__ q_norm,
     const float* __restrict__ k_norm, float eps, float temp_coef, int temp_every, const int* __restrict__ positions,
     const int* __restrict__ slots, T* __restrict__ k_pool, T* __restrict__ v_pool, int q_heads, int k_heads, int dk,
-    int v_heads, int dv, int block_size) {
+    int v_heads, int dv, int block_size, const float* __restrict__ freq, int rot_dims, int unit_norm) {
     const int n = blockIdx.x, lane = threadIdx.x;
     int head = blockIdx.y;
     const float* row = proj + (size_t)n * proj_stride;
@@ -117,9 +129,13 @@ __global__ __launch_bounds__(LLMS_WAVE) void norm_store_kernel(
         const float* src = row + (size_t)head * dk;  // (keys follow the queries)
         const float* w = is_q ? q_norm : k_norm;
         float mul = 1.f;
-        if (w) {
+        const float position = rot_dims > 0 ? (float)positions[n] : 0.f;
+        if (w || unit_norm) {
             float ss = 0.f;
-            for (int d = lane; d < dk; d += LLMS_WAVE) ss = fmaf(src[d], src[d], ss);
+            for (int d = lane; d < dk; d += LLMS_WAVE) {
+                const float x = rot_dims > 0 ? turned_element(src, d, rot_dims, position, freq) : src[d];
+                ss = fmaf(x, x, ss);
+            }
             mul = 1.f / sqrtf(wave_sum(ss) / (float)dk + eps);
         }
         float factor = 1.f;
@@ -135,7 +151,7 @@ __global__ __launch_bounds__(LLMS_WAVE) void norm_store_kernel(
             dst = k_pool + (((size_t)page * k_heads + (head - q_heads)) * block_size + off) * dk;
         }
         for (int d = lane; d < dk; d += LLMS_WAVE) {
-            float x = src[d] * mul;
+            float x = (rot_dims > 0 ? turned_element(src, d, rot_dims, position, freq) : src[d]) * mul;
             if (w) x *= w[d];
             dst[d] = from_f32<T>(x * factor);
         }
@@ -162,6 +178,7 @@ struct ComposedArgs {
     int dist_reach;
     const float* gate;  // 32-bit products [N, gate_stride], or null
     int gate_stride;
+    int sink;  // the softmax's denominator holds one more term, exp(0): a key of score zero that has no value
 };
 
 template <typename T>
@@ -255,6 +272,11 @@ __global__ __launch_bounds__(AC_THREADS) void attend_composed_kernel(
             const float m_new = fmaxf(m, wave_max(sc));
             const float e = v < n_vis ? expf(sc - m_new) : 0.f;
             l = l * expf(m - m_new) + wave_sum(e);
+            m = m_new;
+        }
+        if (a.sink) {
+            const float m_new = fmaxf(m, 0.f);
+            l = l * expf(m - m_new) + expf(-m_new);
             m = m_new;
         }
         if (lane == 0) {
@@ -377,8 +399,10 @@ int llms_conv_store(int dtype, void* q_out, int q_stride, const float* proj, int
 int llms_norm_store(int dtype, void* q_out, int q_stride, const float* proj, int proj_stride, const float* q_norm,
                     const float* k_norm, float eps, float temp_coef, int temp_every, const int* positions, const int* slots,
                     void* k_pool, void* v_pool, int n_tokens, int q_heads, int k_heads, int dk, int v_heads, int dv,
-                    int block_size, hipStream_t stream) {
+                    int block_size, const float* freq, int rot_dims, int unit_norm, hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && q_heads > 0 && k_heads >= 0 && v_heads >= 0 && dk > 0 && dv > 0, "norm_store: sizes must be positive");
+    LLMS_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk && (rot_dims == 0 || (freq && positions)),
+                 "norm_store: an even number of turned dimensions within a head, with frequencies and positions");
     LLMS_REQUIRE(temp_every == 0 || positions, "norm_store: a factor by position needs the positions");
     LLMS_REQUIRE(!slots || (k_pool && v_pool && block_size > 0), "norm_store: slots given without pools");
     LLMS_REQUIRE(q_heads + k_heads + v_heads <= 65535, "norm_store: up to 65,535 heads in all");
@@ -386,11 +410,13 @@ int llms_norm_store(int dtype, void* q_out, int q_stride, const float* proj, int
     if (dtype == 0)
         norm_store_kernel<float><<<grid, LLMS_WAVE, 0, stream>>>((float*)q_out, q_stride, proj, proj_stride, q_norm, k_norm, eps,
                                                                  temp_coef, temp_every, positions, slots, (float*)k_pool,
-                                                                 (float*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size);
+                                                                 (float*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size,
+                                                                 freq, rot_dims, unit_norm);
     else if (dtype == 1)
         norm_store_kernel<bf16><<<grid, LLMS_WAVE, 0, stream>>>((bf16*)q_out, q_stride, proj, proj_stride, q_norm, k_norm, eps,
                                                                 temp_coef, temp_every, positions, slots, (bf16*)k_pool,
-                                                                (bf16*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size);
+                                                                (bf16*)v_pool, q_heads, k_heads, dk, v_heads, dv, block_size,
+                                                                freq, rot_dims, unit_norm);
     else
         LLMS_REQUIRE(false, "norm_store: dtype must be 0 (float32) or 1 (bfloat16)");
     LLMS_LAUNCH_CHECK();
@@ -412,7 +438,8 @@ int llms_attend_composed(int dtype, void* out, int out_stride, const void* q, in
                          int kv_heads, int maps,
                          int dk, int dv, int block_size, int window, int keep_first, int chunk, float scale,
                          const float* slopes, const float* talk, float lambda, int head_norm, float eps, float out_scale,
-                         const float* dist_bias, int dist_reach, const float* gate, int gate_stride, hipStream_t stream) {
+                         const float* dist_bias, int dist_reach, const float* gate, int gate_stride, int sink,
+                         hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && heads > 0 && kv_heads > 0 && dk > 0 && dv > 0, "attend_composed: sizes must be positive");
     LLMS_REQUIRE(!dist_bias || dist_reach >= 0, "attend_composed: a distance table has at least one entry per head");
     LLMS_REQUIRE(heads % kv_heads == 0, "attend_composed: heads must be a multiple of kv_heads");
@@ -427,7 +454,7 @@ int llms_attend_composed(int dtype, void* out, int out_stride, const void* q, in
     a.heads = heads, a.kv_heads = kv_heads, a.maps = maps, a.dk = dk, a.dv = dv, a.block_size = block_size;
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
     a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
-    a.dist_bias = dist_bias, a.dist_reach = dist_reach, a.gate = gate, a.gate_stride = gate_stride;
+    a.dist_bias = dist_bias, a.dist_reach = dist_reach, a.gate = gate, a.gate_stride = gate_stride, a.sink = sink;
     if (dtype == 0) {
         auto kernel = attend_composed_kernel<float>;
         if (lds > 48 * 1024)

@@ -9,15 +9,21 @@
 //                    rotated parts turned into q'[n, h, r ..]
 //   attend_latent    out[n, h, :r] = sum_j softmax_j(q'[n, h] . row_j * scale) c_j over the keys the window allows
 //
-// Rotation: pairs (2i, 2i+1) of the first `dims` numbers of the rotated part, angle position * freq[i], the rest of
-// the part passes.  Norms, angles, scores, softmax and sums are 32-bit; T (float or bfloat16) is what is stored.
+// Rotation: pairs (2i, 2i+1) of the first `dims` numbers of the rotated part (`half`: pairs (i, i + dims/2) instead),
+// angle position * freq[i], the rest of the part passes.  Norms, angles, scores, softmax and sums are 32-bit; T (float or bfloat16) is what is stored.
 #include "common.h"
 
 #define LAT_THREADS 256
 
 __device__ __forceinline__ float rotated_element(const float* __restrict__ part, int e, int dims, float position,
-                                                 const float* __restrict__ freq) {
+                                                 const float* __restrict__ freq, int half = 0) {
     if (e >= dims) return part[e];
+    if (half) {  // dimension i turns together with dimension i + dims / 2
+        const int h = dims >> 1, i = e < h ? e : e - h;
+        const float2 sc = rotary_angle(position, freq[i]);
+        const float2 turned = rotate_pair(part[i], part[i + h], sc.y, sc.x);
+        return e < h ? turned.x : turned.y;
+    }
     const int i = e >> 1;
     const float2 sc = rotary_angle(position, freq[i]);  // (sine, cosine)
     const float2 turned = rotate_pair(part[2 * i], part[2 * i + 1], sc.y, sc.x);
@@ -30,7 +36,7 @@ template <typename T>
 __global__ __launch_bounds__(LAT_THREADS) void latent_prepare_kernel(
     T* __restrict__ cq, T* __restrict__ pool, const float* __restrict__ z, int z_ld, int col_q, int q_rank, int col_c,
     int r, int dr, const float* __restrict__ wq, const float* __restrict__ wc, const float* __restrict__ freq, int dims,
-    const int* __restrict__ positions, const int* __restrict__ slots, float eps) {
+    const int* __restrict__ positions, const int* __restrict__ slots, float eps, int half) {
     __shared__ float red[16];
     const int n = blockIdx.x;
     const float* zr = z + (size_t)n * z_ld;
@@ -51,18 +57,18 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_prepare_kernel(
     for (int c = threadIdx.x; c < r; c += LAT_THREADS) row[c] = from_f32<T>(zr[col_c + c] * inv * wc[c]);
     const float position = (float)positions[n];
     for (int e = threadIdx.x; e < dr; e += LAT_THREADS)
-        row[r + e] = from_f32<T>(rotated_element(zr + col_c + r, e, dims, position, freq));
+        row[r + e] = from_f32<T>(rotated_element(zr + col_c + r, e, dims, position, freq, half));
 }
 
 // grid: tokens.  q [N, H, dn + dr] float -> plain [N, H, dn] and folded[n, h, r + e] (row length H * (r + dr)).
 template <typename T>
 __global__ __launch_bounds__(LAT_THREADS) void latent_query_kernel(
     T* __restrict__ plain, T* __restrict__ folded, const float* __restrict__ q, int heads, int dn, int dr, int r,
-    const float* __restrict__ freq, int dims, const int* __restrict__ positions) {
+    const float* __restrict__ freq, int dims, const int* __restrict__ positions, int half_pairs) {
     const int n = blockIdx.x, dq = dn + dr;
     const float position = (float)positions[n];
     const float* qr = q + (size_t)n * heads * dq;
-    if (dn % 2 == 0 && dr % 2 == 0) {  // a thread takes two neighbours: a pair of the rotation has one sine and cosine
+    if (dn % 2 == 0 && dr % 2 == 0 && !half_pairs) {  // a thread takes two neighbours: a pair of the rotation has one sine and cosine
         const int half = dq / 2;
         for (int i = threadIdx.x; i < heads * half; i += LAT_THREADS) {
             const int h = i / half, e = 2 * (i - h * half);
@@ -88,7 +94,7 @@ __global__ __launch_bounds__(LAT_THREADS) void latent_query_kernel(
             plain[((size_t)n * heads + h) * dn + e] = from_f32<T>(qr[i]);
         else
             folded[((size_t)n * heads + h) * (r + dr) + r + (e - dn)] =
-                from_f32<T>(rotated_element(qr + h * dq + dn, e - dn, dims, position, freq));
+                from_f32<T>(rotated_element(qr + h * dq + dn, e - dn, dims, position, freq, half_pairs));
     }
 }
 
@@ -177,30 +183,30 @@ extern "C" {
 
 int llms_latent_prepare(int dtype, void* cq, void* pool, const float* z, int z_ld, int col_q, int q_rank, int col_c, int r,
                         int dr, const float* wq, const float* wc, const float* freq, int dims, const int* positions,
-                        const int* slots, float eps, int n, hipStream_t stream) {
+                        const int* slots, float eps, int n, int half_pairs, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && r > 0 && dr >= 0 && q_rank >= 0, "latent_prepare: sizes must be positive");
     LLMS_REQUIRE(dims >= 0 && dims <= dr && dims % 2 == 0, "latent_prepare: an even number of turned dimensions within the part");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "latent_prepare: dtype must be 0 (float32) or 1 (bfloat16)");
     if (dtype == 0)
         latent_prepare_kernel<float><<<n, LAT_THREADS, 0, stream>>>((float*)cq, (float*)pool, z, z_ld, col_q, q_rank, col_c, r, dr,
-                                                                    wq, wc, freq, dims, positions, slots, eps);
+                                                                    wq, wc, freq, dims, positions, slots, eps, half_pairs);
     else
         latent_prepare_kernel<bf16><<<n, LAT_THREADS, 0, stream>>>((bf16*)cq, (bf16*)pool, z, z_ld, col_q, q_rank, col_c, r, dr,
-                                                                   wq, wc, freq, dims, positions, slots, eps);
+                                                                   wq, wc, freq, dims, positions, slots, eps, half_pairs);
     LLMS_LAUNCH_CHECK();
 }
 
 int llms_latent_query(int dtype, void* plain, void* folded, const float* q, int heads, int dn, int dr, int r,
-                      const float* freq, int dims, const int* positions, int n, hipStream_t stream) {
+                      const float* freq, int dims, const int* positions, int n, int half_pairs, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && heads > 0 && dn > 0 && dr >= 0 && r > 0, "latent_query: sizes must be positive");
     LLMS_REQUIRE(dims >= 0 && dims <= dr && dims % 2 == 0, "latent_query: an even number of turned dimensions within the part");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "latent_query: dtype must be 0 (float32) or 1 (bfloat16)");
     if (dtype == 0)
         latent_query_kernel<float><<<n, LAT_THREADS, 0, stream>>>((float*)plain, (float*)folded, q, heads, dn, dr, r, freq, dims,
-                                                                  positions);
+                                                                  positions, half_pairs);
     else
         latent_query_kernel<bf16><<<n, LAT_THREADS, 0, stream>>>((bf16*)plain, (bf16*)folded, q, heads, dn, dr, r, freq, dims,
-                                                                 positions);
+                                                                 positions, half_pairs);
     LLMS_LAUNCH_CHECK();
 }
 

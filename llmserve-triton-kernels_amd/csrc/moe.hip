@@ -2,7 +2,8 @@
 //   moe_router    z = W_router h in 32-bit, s = sigmoid(z) or softmax(z) over all experts, the `top` largest (the lower expert
 //                 wins a tie), in descending order; weight = score or score / (sum of the chosen scores + renorm_eps).
 //                 With `groups` > 1 the experts form that many equal groups of neighbours, a group's score is its largest
-//                 score, and only experts of the `keep` best groups (the lower group wins a tie) can be chosen
+//                 score, and only experts of the `keep` best groups (the lower group wins a tie) can be chosen.
+//                 `bias` is added to z; `extra` rows of W_router behind the experts' give extra_out = their products
 //   moe_rank      for expert e: how many (token, choice) pairs chose it, and each such pair's rank among them in the
 //                 order of the pairs (so the sorted order is stable and the same whatever runs beside it)
 //   moe_offsets   seg[e] = pairs of all experts before e, tile_start[e] = tiles of rows of all experts before e
@@ -20,12 +21,13 @@
 template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
     int* __restrict__ chosen, float* __restrict__ weight, const T* __restrict__ h, const T* __restrict__ w_router,
-    int hidden, int experts, int top, int renormalize, int softmax, int groups, int keep, float renorm_eps) {
+    int hidden, int experts, int top, int renormalize, int softmax, int groups, int keep, float renorm_eps,
+    const float* __restrict__ bias, int extra, float* __restrict__ extra_out) {
     extern __shared__ float score[];  // experts, then groups
     const int n = blockIdx.x, lane = threadIdx.x % LLMS_WAVE, wave = threadIdx.x / LLMS_WAVE;
     const T* row = h + (size_t)n * hidden;
     const bool vec = hidden % (16 / sizeof(T)) == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)w_router % 16) == 0;
-    for (int e = wave; e < experts; e += MOE_THREADS / LLMS_WAVE) {
+    for (int e = wave; e < experts + extra; e += MOE_THREADS / LLMS_WAVE) {
         const T* wr = w_router + (size_t)e * hidden;
         float dot = 0.f;
         if (vec) {  // 16 bytes a lane and load, four loads in flight
@@ -52,6 +54,11 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_router_kernel(
             for (int c = lane; c < hidden; c += LLMS_WAVE) dot = fmaf(to_f32(row[c]), to_f32(wr[c]), dot);
         }
         dot = wave_sum(dot);
+        if (e >= experts) {  // rows of the weight behind the experts': their products leave as they are
+            if (lane == 0) extra_out[(size_t)n * extra + (e - experts)] = dot;
+            continue;
+        }
+        if (bias) dot += bias[e];
         // (a row that is not a number, as a padding row may be, gets a score like any other: every choice below must
         // name an expert that exists)
         if (lane == 0) score[e] = dot == dot ? (softmax ? dot : 1.f / (1.f + expf(-dot))) : 0.f;
@@ -264,9 +271,14 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_place_few_kernel(
 __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restrict__ y, const float* __restrict__ rows,
                                                                   const int* __restrict__ place, int hidden, int top,
                                                                   int parts, long part_stride,
-                                                                  const float* __restrict__ weight) {
+                                                                  const float* __restrict__ weight,
+                                                                  const float* __restrict__ always,
+                                                                  const float* __restrict__ always_gate) {
     const int n = blockIdx.x;
-    if (hidden % 4 == 0 && part_stride % 4 == 0 && ((uintptr_t)rows % 16) == 0 && ((uintptr_t)y % 16) == 0) {
+    float always_w = 0.f;  // what every token adds beside its choices: sigmoid(gate[n]) * always[n] (gate null: 1)
+    if (always) always_w = always_gate ? 1.f / (1.f + expf(-always_gate[n])) : 1.f;
+    if (hidden % 4 == 0 && part_stride % 4 == 0 && ((uintptr_t)rows % 16) == 0 && ((uintptr_t)y % 16) == 0 &&
+        ((uintptr_t)always % 16) == 0) {
         // 16 bytes a thread and load, the loads of four summands in flight together
         for (int c = 4 * threadIdx.x; c < hidden; c += 4 * MOE_THREADS) {
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -292,6 +304,11 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
                     }
                 }
             }
+            if (always) {
+                const float4 a = *reinterpret_cast<const float4*>(always + (size_t)n * hidden + c);
+                v.x = fmaf(always_w, a.x, v.x), v.y = fmaf(always_w, a.y, v.y);
+                v.z = fmaf(always_w, a.z, v.z), v.w = fmaf(always_w, a.w, v.w);
+            }
             *reinterpret_cast<float4*>(y + (size_t)n * hidden + c) = v;
         }
         return;
@@ -303,6 +320,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
             const float wk = weight ? weight[(size_t)n * top + k] : 1.f;
             for (int p = 0; p < parts; ++p) v = weight ? fmaf(wk, row[(size_t)p * part_stride], v) : v + row[(size_t)p * part_stride];
         }
+        if (always) v = fmaf(always_w, always[(size_t)n * hidden + c], v);
         y[(size_t)n * hidden + c] = v;
     }
 }
@@ -310,8 +328,10 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_combine_kernel(float* __restr
 extern "C" {
 
 int llms_moe_router(int dtype, int* chosen, float* weight, const void* h, const void* w_router, int n, int hidden, int experts,
-                    int top, int renormalize, int softmax, int groups, int keep, float renorm_eps, hipStream_t stream) {
+                    int top, int renormalize, int softmax, int groups, int keep, float renorm_eps, const float* bias, int extra,
+                    float* extra_out, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && hidden > 0 && experts > 0, "moe_router: sizes must be positive");
+    LLMS_REQUIRE(extra >= 0 && (extra == 0 || extra_out), "moe_router: extra rows need a place for their products");
     LLMS_REQUIRE(top >= 1 && top <= MOE_MAX_TOP && top <= experts, "moe_router: 1 to 16 choices, no more than there are experts");
     LLMS_REQUIRE(experts <= 8192, "moe_router: up to 8,192 experts");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "moe_router: dtype must be 0 (float32) or 1 (bfloat16)");
@@ -321,10 +341,10 @@ int llms_moe_router(int dtype, int* chosen, float* weight, const void* h, const 
     const size_t lds = (size_t)(experts + groups) * sizeof(float);
     if (dtype == 0)
         moe_router_kernel<float><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const float*)h, (const float*)w_router, hidden,
-                                                                  experts, top, renormalize, softmax, groups, keep, renorm_eps);
+                                                                  experts, top, renormalize, softmax, groups, keep, renorm_eps, bias, extra, extra_out);
     else
         moe_router_kernel<bf16><<<n, MOE_THREADS, lds, stream>>>(chosen, weight, (const bf16*)h, (const bf16*)w_router, hidden,
-                                                                 experts, top, renormalize, softmax, groups, keep, renorm_eps);
+                                                                 experts, top, renormalize, softmax, groups, keep, renorm_eps, bias, extra, extra_out);
     LLMS_LAUNCH_CHECK();
 }
 
@@ -369,9 +389,9 @@ int llms_moe_place_few(int dtype, void* xs, int* place, int* seg, int* tile_star
 }
 
 int llms_moe_combine(float* y, const float* rows, const int* place, int n, int hidden, int top, int parts, long part_stride,
-                     const float* weight, hipStream_t stream) {
+                     const float* weight, const float* always, const float* always_gate, hipStream_t stream) {
     LLMS_REQUIRE(n > 0 && hidden > 0 && top > 0 && parts > 0, "moe_combine: sizes must be positive");
-    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top, parts, part_stride, weight);
+    moe_combine_kernel<<<n, MOE_THREADS, 0, stream>>>(y, rows, place, hidden, top, parts, part_stride, weight, always, always_gate);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -1,0 +1,351 @@
+// Recurrent mixers over a state of fixed size per request, everything in 32-bit:
+//
+//   conv_act        a short causal convolution per channel over the 32-bit products of a step's tokens, plus a bias,
+//                   then SiLU: y_t = act(b + sum_j w[c, j] u_(t - taps + 1 + j)), zeros before the sequence.  A request's
+//                   last taps - 1 input rows are a ring in its state, indexed by position, so a portion of any length
+//                   reads what it needs.  The result leaves as 32-bit and, where asked for, rounded to T as well.
+//   conv_ring       the ring takes the last taps - 1 input rows of every request of the step (a launch of its own,
+//                   because a token's write would race with its neighbours' reads; when every request brings one
+//                   token, conv_act writes the ring itself).
+//   selective_scan  per channel c and state n:  S <- exp(dt_c A[c, n]) S + dt_c x_c B_n,  y_c = sum_n S C_n + D_c x_c,
+//                   dt = softplus(dt_raw + bias), and y silu(z) leaves rounded once.  16 lanes share a channel's states.
+//   unit_heads      every head of q and k is divided by sqrt(sum of squares + eps); q is multiplied by a factor.
+//   delta_scan      the gated delta rule per head over a state S [dk, dv]:
+//                   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the token's write)
+//                   with beta = sigmoid(zb) and g = exp(-exp(A_log) softplus(za + dt_bias)).  16 lanes share a column.
+//   delta_finish    each head of o is divided by its root mean square (eps inside the root), multiplied by a weight
+//                   that all heads share and by silu(gate), rounded once.
+//
+// A request of length 0 is padding: nothing of it is read or written.  The state of request b lies at
+// state + state_slots[b] * slot_stride (+ an offset per kind of state); a portion starts from it and leaves it behind
+// its last token, so any cut of a prompt gives the same recurrence.
+#include "common.h"
+
+#define RC_THREADS 256
+
+__device__ __forceinline__ float rc_silu(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float rc_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// sum over the 16 lanes of a row of the wave, the same value in all of them (no LDS: four lane exchanges inside the row)
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xF, 0xF, true));  // row_half_mirror
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xF, 0xF, true));  // row_mirror
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------- convolution
+// grid (tokens, channel blocks).  u [N, u_ld] columns u_col ..; ring [taps - 1, channels] at ring_off inside a slot.
+template <typename T>
+__global__ __launch_bounds__(RC_THREADS) void conv_act_kernel(
+    float* __restrict__ y32, int y32_ld, T* __restrict__ y16, int y16_ld, const float* __restrict__ u, int u_ld, int u_col,
+    const float* __restrict__ taps_w, const float* __restrict__ bias, int taps, int channels, float* __restrict__ state,
+    size_t slot_stride, size_t ring_off, const int* __restrict__ state_slots, const int* __restrict__ token_seq,
+    const int* __restrict__ positions, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
+    int activation, int update) {
+    const int n = blockIdx.x;
+    const int c = blockIdx.y * RC_THREADS + threadIdx.x;
+    if (c >= channels) return;
+    const int b = token_seq[n];
+    if (context_lens[b] <= 0) return;
+    const int p = positions[n];
+    const int first_row = cu_seqlens[b];
+    const int first_pos = p - (n - first_row);
+    float* ring = taps > 1 ? state + (size_t)state_slots[b] * slot_stride + ring_off : nullptr;
+    float y = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int pos = p - (taps - 1) + j;
+        float v = 0.f;
+        if (pos >= first_pos)
+            v = u[(size_t)(first_row + pos - first_pos) * u_ld + u_col + c];
+        else if (pos >= 0)
+            v = ring[(size_t)(pos % (taps - 1)) * channels + c];
+        y = fmaf(taps_w[(size_t)c * taps + j], v, y);
+    }
+    if (update && taps > 1)  // (every request brings one token: nobody else reads this ring, and this thread has read its place)
+        ring[(size_t)(p % (taps - 1)) * channels + c] = u[(size_t)n * u_ld + u_col + c];
+    if (activation) y = rc_silu(y);
+    if (y32) y32[(size_t)n * y32_ld + c] = y;
+    if (y16) y16[(size_t)n * y16_ld + c] = from_f32<T>(y);
+}
+
+// grid (requests, channel blocks)
+__global__ __launch_bounds__(RC_THREADS) void conv_ring_kernel(
+    float* __restrict__ state, size_t slot_stride, size_t ring_off, const int* __restrict__ state_slots,
+    const float* __restrict__ u, int u_ld, int u_col, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ context_lens, int taps, int channels) {
+    const int b = blockIdx.x;
+    const int c = blockIdx.y * RC_THREADS + threadIdx.x;
+    if (c >= channels) return;
+    const int first_row = cu_seqlens[b], count = cu_seqlens[b + 1] - first_row;
+    const int end = context_lens[b];
+    if (count <= 0 || end <= 0) return;
+    const int first_pos = end - count;
+    float* ring = state + (size_t)state_slots[b] * slot_stride + ring_off;
+    int pos = end - (taps - 1);
+    if (pos < first_pos) pos = first_pos;
+    for (; pos < end; ++pos)
+        ring[(size_t)(pos % (taps - 1)) * channels + c] = u[(size_t)(first_row + pos - first_pos) * u_ld + u_col + c];
+}
+
+// ------------------------------------------------------------------------------------------- selective scan
+// grid (requests, channels / 16).  Thread (channel, lane of 16): states lane, lane + 16, ...  R = ceil(states / 16).
+// x [N, x_ld] (after the convolution), z [N, z_ld] columns z_col .., low [N, low_ld]: B at b_col, C at c_col,
+// dt_raw [N, dt_ld]; S [channels, states] at scan_off inside a slot.
+template <typename T, int R>
+__global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
+    T* __restrict__ out, int out_ld, const float* __restrict__ x, int x_ld, const float* __restrict__ z, int z_ld, int z_col,
+    const float* __restrict__ low, int low_ld, int b_col, int c_col, const float* __restrict__ dt_raw, int dt_ld,
+    const float* __restrict__ dt_bias, const float* __restrict__ a_neg, const float* __restrict__ d_skip, int channels,
+    int states, float* __restrict__ state, size_t slot_stride, size_t scan_off, const int* __restrict__ state_slots,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens) {
+    const int b = blockIdx.x;
+    const int lane = threadIdx.x & 15;
+    const int c = blockIdx.y * (RC_THREADS / 16) + (threadIdx.x >> 4);
+    const int first_row = cu_seqlens[b], count = cu_seqlens[b + 1] - first_row;
+    if (count <= 0 || context_lens[b] <= 0) return;
+    const bool live = c < channels;
+    const int cc = live ? c : channels - 1;  // (lanes beyond the last channel compute along and store nothing)
+    float* srow = state + (size_t)state_slots[b] * slot_stride + scan_off + (size_t)cc * states;
+    float s[R], a[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int k = lane + 16 * r;
+        s[r] = k < states ? srow[k] : 0.f;
+        a[r] = k < states ? a_neg[(size_t)cc * states + k] : 0.f;
+    }
+    const float bias = dt_bias[cc], skip = d_skip[cc];
+    for (int t = 0; t < count; ++t) {
+        const size_t row = (size_t)(first_row + t);
+        const float dt = rc_softplus(dt_raw[row * dt_ld + cc] + bias);
+        const float xv = x[row * x_ld + cc];
+        const float dx = dt * xv;
+        float y = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int k = lane + 16 * r;
+            const float bn = k < states ? low[row * low_ld + b_col + k] : 0.f;
+            const float cn = k < states ? low[row * low_ld + c_col + k] : 0.f;
+            s[r] = fmaf(expf(dt * a[r]), s[r], dx * bn);
+            y = fmaf(s[r], cn, y);
+        }
+        y = row16_sum(y);
+        if (lane == 0 && live) {
+            y = fmaf(skip, xv, y);
+            out[row * out_ld + c] = from_f32<T>(y * rc_silu(z[row * z_ld + z_col + c]));
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int k = lane + 16 * r;
+            if (k < states) srow[k] = s[r];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------- unit heads
+// grid (tokens, heads of q + heads of k): one wave a head, in place on x [N, ld]: q heads at q_col, k heads behind them at k_col
+__global__ __launch_bounds__(LLMS_WAVE) void unit_heads_kernel(float* __restrict__ x, int ld, int q_col, int k_col, int q_heads,
+                                                               int k_heads, int dk, float eps, float q_factor) {
+    const int n = blockIdx.x, lane = threadIdx.x;
+    const int head = blockIdx.y;
+    const bool is_q = head < q_heads;
+    float* v = x + (size_t)n * ld + (is_q ? q_col + head * dk : k_col + (head - q_heads) * dk);
+    float ss = 0.f;
+    for (int d = lane; d < dk; d += LLMS_WAVE) ss = fmaf(v[d], v[d], ss);
+    const float mul = (is_q ? q_factor : 1.f) / sqrtf(wave_sum(ss) + eps);
+    for (int d = lane; d < dk; d += LLMS_WAVE) v[d] *= mul;
+}
+
+// ------------------------------------------------------------------------------------------- delta rule
+// grid (requests, heads, columns / 16).  Thread (column j, lane of 16): rows lane, lane + 16, ... of column j of S.
+// qkv [N, qkv_ld]: q heads at q_col (kv_heads * dk), k heads at k_col, v heads at v_col (heads * dv), prepared;
+// gates [N, g_ld]: za at a_col + head, zb at b_col + head.  S [heads, dk, dv] at scan_off inside a slot.
+template <int R>
+__global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
+    float* __restrict__ o, int o_ld, const float* __restrict__ qkv, int qkv_ld, int q_col, int k_col, int v_col,
+    const float* __restrict__ gates, int g_ld, int a_col, int b_col, const float* __restrict__ a_log,
+    const float* __restrict__ dt_bias, int heads, int kv_heads, int dk, int dv, float* __restrict__ state, size_t slot_stride,
+    size_t scan_off, const int* __restrict__ state_slots, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ context_lens) {
+    const int b = blockIdx.x, h = blockIdx.y;
+    const int lane = threadIdx.x & 15;
+    const int j = blockIdx.z * (RC_THREADS / 16) + (threadIdx.x >> 4);
+    const int first_row = cu_seqlens[b], count = cu_seqlens[b + 1] - first_row;
+    if (count <= 0 || context_lens[b] <= 0) return;
+    const bool live = j < dv;
+    const int jj = live ? j : dv - 1;
+    const int g = h / (heads / kv_heads);
+    float* sh = state + (size_t)state_slots[b] * slot_stride + scan_off + (size_t)h * dk * dv;
+    float s[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int i = lane + 16 * r;
+        s[r] = i < dk ? sh[(size_t)i * dv + jj] : 0.f;
+    }
+    const float rate = expf(a_log[h]), bias = dt_bias[h];
+    for (int t = 0; t < count; ++t) {
+        const size_t row = (size_t)(first_row + t);
+        const float* qr = qkv + row * qkv_ld + q_col + g * dk;
+        const float* kr = qkv + row * qkv_ld + k_col + g * dk;
+        float kk[R], qq[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = lane + 16 * r;
+            kk[r] = i < dk ? kr[i] : 0.f;
+            qq[r] = i < dk ? qr[i] : 0.f;
+        }
+        const float v = qkv[row * qkv_ld + v_col + h * dv + jj];
+        const float decay = expf(-rate * rc_softplus(gates[row * g_ld + a_col + h] + bias));
+        const float beta = 1.f / (1.f + expf(-gates[row * g_ld + b_col + h]));
+        // with S' = decay S:  u = beta (v - S'^T k),  o = (S' + k u^T)^T q = S'^T q + (k . q) u
+        float sk = 0.f, sq = 0.f, kq = 0.f;
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            s[r] *= decay;
+            sk = fmaf(s[r], kk[r], sk);
+            sq = fmaf(s[r], qq[r], sq);
+            kq = fmaf(kk[r], qq[r], kq);
+        }
+        sk = row16_sum(sk), sq = row16_sum(sq), kq = row16_sum(kq);
+        const float u = beta * (v - sk);
+#pragma unroll
+        for (int r = 0; r < R; ++r) s[r] = fmaf(kk[r], u, s[r]);
+        if (lane == 0 && live) o[row * o_ld + h * dv + j] = fmaf(kq, u, sq);
+    }
+    if (live) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int i = lane + 16 * r;
+            if (i < dk) sh[(size_t)i * dv + j] = s[r];
+        }
+    }
+}
+
+// grid (tokens, heads): one wave a head
+template <typename T>
+__global__ __launch_bounds__(LLMS_WAVE) void delta_finish_kernel(T* __restrict__ out, int out_ld, const float* __restrict__ o,
+                                                                 int o_ld, const float* __restrict__ gate, int gate_ld,
+                                                                 int gate_col, const float* __restrict__ weight, int dv,
+                                                                 float eps) {
+    const int n = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* v = o + (size_t)n * o_ld + (size_t)h * dv;
+    float ss = 0.f;
+    for (int d = lane; d < dv; d += LLMS_WAVE) ss = fmaf(v[d], v[d], ss);
+    const float mul = 1.f / sqrtf(wave_sum(ss) / (float)dv + eps);
+    for (int d = lane; d < dv; d += LLMS_WAVE) {
+        const float z = gate[(size_t)n * gate_ld + gate_col + h * dv + d];
+        out[(size_t)n * out_ld + h * dv + d] = from_f32<T>(v[d] * mul * weight[d] * rc_silu(z));
+    }
+}
+
+extern "C" {
+
+int llms_conv_act(int dtype, float* y32, int y32_ld, void* y16, int y16_ld, const float* u, int u_ld, int u_col,
+                  const float* taps_w, const float* bias, int taps, int channels, float* state, size_t slot_stride,
+                  size_t ring_off, const int* state_slots, const int* token_seq, const int* positions, const int* cu_seqlens,
+                  const int* context_lens, int n_tokens, int activation, int update, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && channels > 0 && taps >= 1, "conv_act: sizes must be positive");
+    LLMS_REQUIRE(u && taps_w && token_seq && positions && cu_seqlens && context_lens, "conv_act: a needed operand is missing");
+    LLMS_REQUIRE(taps == 1 || (state && state_slots), "conv_act: two taps or more need the state");
+    LLMS_REQUIRE(y32 || y16, "conv_act: nothing to store");
+    dim3 grid(n_tokens, (channels + RC_THREADS - 1) / RC_THREADS);
+    if (dtype == 0)
+        conv_act_kernel<float><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (float*)y16, y16_ld, u, u_ld, u_col, taps_w, bias,
+                                                                taps, channels, state, slot_stride, ring_off, state_slots,
+                                                                token_seq, positions, cu_seqlens, context_lens, activation, update);
+    else if (dtype == 1)
+        conv_act_kernel<bf16><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (bf16*)y16, y16_ld, u, u_ld, u_col, taps_w, bias,
+                                                               taps, channels, state, slot_stride, ring_off, state_slots,
+                                                               token_seq, positions, cu_seqlens, context_lens, activation, update);
+    else
+        LLMS_REQUIRE(false, "conv_act: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_conv_ring(float* state, size_t slot_stride, size_t ring_off, const int* state_slots, const float* u, int u_ld,
+                   int u_col, const int* cu_seqlens, const int* context_lens, int n_seqs, int taps, int channels,
+                   hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && taps > 1 && channels > 0, "conv_ring: sizes must be positive and taps at least 2");
+    dim3 grid(n_seqs, (channels + RC_THREADS - 1) / RC_THREADS);
+    conv_ring_kernel<<<grid, RC_THREADS, 0, stream>>>(state, slot_stride, ring_off, state_slots, u, u_ld, u_col, cu_seqlens,
+                                                      context_lens, taps, channels);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_selective_scan(int dtype, void* out, int out_ld, const float* x, int x_ld, const float* z, int z_ld, int z_col,
+                        const float* low, int low_ld, int b_col, int c_col, const float* dt_raw, int dt_ld,
+                        const float* dt_bias, const float* a_neg, const float* d_skip, int channels, int states, float* state,
+                        size_t slot_stride, size_t scan_off, const int* state_slots, const int* cu_seqlens,
+                        const int* context_lens, int n_seqs, hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && channels > 0 && states > 0 && states <= 256, "selective_scan: 1 to 256 states per channel");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "selective_scan: dtype must be 0 (float32) or 1 (bfloat16)");
+    dim3 grid(n_seqs, (channels + RC_THREADS / 16 - 1) / (RC_THREADS / 16));
+    const int r = (states + 15) / 16;
+#define SCAN_GO(T, R)                                                                                                     \
+    selective_scan_kernel<T, R><<<grid, RC_THREADS, 0, stream>>>((T*)out, out_ld, x, x_ld, z, z_ld, z_col, low, low_ld, b_col, \
+                                                                 c_col, dt_raw, dt_ld, dt_bias, a_neg, d_skip, channels,  \
+                                                                 states, state, slot_stride, scan_off, state_slots,      \
+                                                                 cu_seqlens, context_lens)
+#define SCAN_R(R)                                                                                                         \
+    do {                                                                                                                  \
+        if (dtype == 0) SCAN_GO(float, R);                                                                                \
+        else SCAN_GO(bf16, R);                                                                                            \
+    } while (0)
+    if (r <= 1) SCAN_R(1);
+    else if (r <= 2) SCAN_R(2);
+    else if (r <= 4) SCAN_R(4);
+    else if (r <= 8) SCAN_R(8);
+    else SCAN_R(16);
+#undef SCAN_R
+#undef SCAN_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_unit_heads(float* x, int ld, int q_col, int k_col, int q_heads, int k_heads, int dk, float eps, float q_factor,
+                    int n_tokens, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && q_heads >= 0 && k_heads >= 0 && q_heads + k_heads > 0 && dk > 0, "unit_heads: sizes must be positive");
+    LLMS_REQUIRE(q_heads + k_heads <= 65535, "unit_heads: up to 65,535 heads in all");
+    dim3 grid(n_tokens, q_heads + k_heads);
+    unit_heads_kernel<<<grid, LLMS_WAVE, 0, stream>>>(x, ld, q_col, k_col, q_heads, k_heads, dk, eps, q_factor);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_delta_scan(float* o, int o_ld, const float* qkv, int qkv_ld, int q_col, int k_col, int v_col, const float* gates,
+                    int g_ld, int a_col, int b_col, const float* a_log, const float* dt_bias, int heads, int kv_heads, int dk,
+                    int dv, float* state, size_t slot_stride, size_t scan_off, const int* state_slots, const int* cu_seqlens,
+                    const int* context_lens, int n_seqs, hipStream_t stream) {
+    LLMS_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta_scan: heads must be a multiple of kv_heads");
+    LLMS_REQUIRE(dk > 0 && dk <= 256 && dv > 0, "delta_scan: keys of 1 to 256 numbers");
+    LLMS_REQUIRE(heads <= 65535, "delta_scan: up to 65,535 heads");
+    dim3 grid(n_seqs, heads, (dv + RC_THREADS / 16 - 1) / (RC_THREADS / 16));
+    const int r = (dk + 15) / 16;
+#define DELTA_GO(R)                                                                                                       \
+    delta_scan_kernel<R><<<grid, RC_THREADS, 0, stream>>>(o, o_ld, qkv, qkv_ld, q_col, k_col, v_col, gates, g_ld, a_col, b_col, \
+                                                          a_log, dt_bias, heads, kv_heads, dk, dv, state, slot_stride,    \
+                                                          scan_off, state_slots, cu_seqlens, context_lens)
+    if (r <= 1) DELTA_GO(1);
+    else if (r <= 2) DELTA_GO(2);
+    else if (r <= 4) DELTA_GO(4);
+    else if (r <= 8) DELTA_GO(8);
+    else DELTA_GO(16);
+#undef DELTA_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_delta_finish(int dtype, void* out, int out_ld, const float* o, int o_ld, const float* gate, int gate_ld, int gate_col,
+                      const float* weight, int heads, int dv, float eps, int n_tokens, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && heads > 0 && heads <= 65535 && dv > 0, "delta_finish: sizes must be positive");
+    dim3 grid(n_tokens, heads);
+    if (dtype == 0)
+        delta_finish_kernel<float><<<grid, LLMS_WAVE, 0, stream>>>((float*)out, out_ld, o, o_ld, gate, gate_ld, gate_col, weight, dv, eps);
+    else if (dtype == 1)
+        delta_finish_kernel<bf16><<<grid, LLMS_WAVE, 0, stream>>>((bf16*)out, out_ld, o, o_ld, gate, gate_ld, gate_col, weight, dv, eps);
+    else
+        LLMS_REQUIRE(false, "delta_finish: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
+}  // extern "C"

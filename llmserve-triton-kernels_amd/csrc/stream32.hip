@@ -8,6 +8,9 @@
 //                    the sublayer before and its coefficients, new_t = sum_s mix[s, t] x_s + out[t] y for all t at
 //                    once; u = sum_t read[t] new_t; out = (u - mean) / sqrt(var + eps) * w (layer norm, no bias; the
 //                    variance is the mean squared deviation).                       (x, y, coefficients float; out T)
+//   normed_add_norm  a sublayer's result joins the stream through a norm of its own, and the next sublayer's input is
+//                    formed in the same pass: x += y / sqrt(mean(y^2) + eps) * wb; out = x / sqrt(mean(x^2) + eps) * w
+//   add_vector       x[n] += v for every row
 // T is float or bfloat16.  One workgroup per row; every reduction has an order fixed by the sizes alone.
 #include "common.h"
 
@@ -427,6 +430,67 @@ __global__ void weighted_sum_kernel(float* out, const float* a, const float* b, 
     if (i < total) out[i] = fmaf(sa, a[i], sb * b[i]);
 }
 
+// grid: rows.  Dynamic LDS: hidden floats (the summed row).  `y` null: nothing joins; `out` null: the sum alone.
+template <typename T>
+__global__ __launch_bounds__(S32_THREADS) void normed_add_norm_kernel(T* __restrict__ out, float* __restrict__ x,
+                                                                      const float* __restrict__ y, const float* __restrict__ wb,
+                                                                      const float* __restrict__ w, const int* __restrict__ rows,
+                                                                      int hidden, float eps_y, float eps, int store) {
+    extern __shared__ float summed[];
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+    float* xr = x + src * hidden;
+    const float* yr = y ? y + src * hidden : nullptr;
+    const bool vec = hidden % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)wb % 16) == 0;
+    float inv_y = 0.f;
+    if (yr) {
+        float ss = 0.f;
+        if (vec) {
+            for (int c = 4 * threadIdx.x; c < hidden; c += 4 * S32_THREADS) {
+                const float4 v = *reinterpret_cast<const float4*>(yr + c);
+                ss = fmaf(v.x, v.x, ss), ss = fmaf(v.y, v.y, ss), ss = fmaf(v.z, v.z, ss), ss = fmaf(v.w, v.w, ss);
+            }
+        } else {
+            for (int c = threadIdx.x; c < hidden; c += S32_THREADS) ss = fmaf(yr[c], yr[c], ss);
+        }
+        inv_y = 1.f / sqrtf(block_sum(ss, red) / (float)hidden + eps_y);
+    }
+    float ss = 0.f;
+    if (vec) {
+        for (int c = 4 * threadIdx.x; c < hidden; c += 4 * S32_THREADS) {
+            float4 v = *reinterpret_cast<const float4*>(xr + c);
+            if (yr) {
+                const float4 a = *reinterpret_cast<const float4*>(yr + c);
+                const float4 b = *reinterpret_cast<const float4*>(wb + c);
+                v.x += a.x * inv_y * b.x, v.y += a.y * inv_y * b.y, v.z += a.z * inv_y * b.z, v.w += a.w * inv_y * b.w;
+                if (store) *reinterpret_cast<float4*>(xr + c) = v;
+            }
+            *reinterpret_cast<float4*>(summed + c) = v;
+            ss = fmaf(v.x, v.x, ss), ss = fmaf(v.y, v.y, ss), ss = fmaf(v.z, v.z, ss), ss = fmaf(v.w, v.w, ss);
+        }
+    } else {
+        for (int c = threadIdx.x; c < hidden; c += S32_THREADS) {
+            float v = xr[c];
+            if (yr) {
+                v += yr[c] * inv_y * wb[c];
+                if (store) xr[c] = v;
+            }
+            summed[c] = v;
+            ss = fmaf(v, v, ss);
+        }
+    }
+    if (!out) return;
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)hidden + eps);
+    T* orow = out + (size_t)r * hidden;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) orow[c] = from_f32<T>(summed[c] * inv * w[c]);
+}
+
+__global__ __launch_bounds__(S32_THREADS) void add_vector_kernel(float* __restrict__ x, const float* __restrict__ v, int hidden) {
+    float* xr = x + (size_t)blockIdx.x * hidden;
+    for (int c = threadIdx.x; c < hidden; c += S32_THREADS) xr[c] += v[c];
+}
+
 extern "C" {
 
 int llms_weighted_sum(float* out, const float* a, const float* b, float sa, float sb, size_t total, hipStream_t stream) {
@@ -562,6 +626,32 @@ int llms_streams_norm(int dtype, void* out, float* x_dst, const float* x_src, in
     else if (dtype == 0) STREAMS_GO(streams_norm_kernel, float);
     else STREAMS_GO(streams_norm_kernel, bf16);
 #undef STREAMS_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_normed_add_norm(int dtype, void* out, float* x, const float* y, const float* wb, const float* w, const int* rows,
+                         int n_out, int hidden, float eps_y, float eps, int store, hipStream_t stream) {
+    LLMS_REQUIRE(n_out > 0 && hidden > 0, "normed_add_norm: sizes must be positive");
+    LLMS_REQUIRE(dtype == 0 || dtype == 1, "normed_add_norm: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_REQUIRE(x && (!y || wb) && (!out || w), "normed_add_norm: a needed operand is missing");
+    LLMS_REQUIRE((size_t)hidden * 4 <= 128 * 1024, "normed_add_norm: a row of up to 32,768 elements");
+    const size_t lds = (size_t)hidden * sizeof(float);
+#define NAN_GO(T)                                                                                                         \
+    do {                                                                                                                  \
+        if (lds > 32 * 1024)                                                                                              \
+            LLMS_HIP_CHECK(hipFuncSetAttribute((const void*)normed_add_norm_kernel<T>,                                    \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));                    \
+        normed_add_norm_kernel<T><<<n_out, S32_THREADS, lds, stream>>>((T*)out, x, y, wb, w, rows, hidden, eps_y, eps, store); \
+    } while (0)
+    if (dtype == 0) NAN_GO(float);
+    else NAN_GO(bf16);
+#undef NAN_GO
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_add_vector(float* x, const float* v, int n, int hidden, hipStream_t stream) {
+    LLMS_REQUIRE(n > 0 && hidden > 0, "add_vector: sizes must be positive");
+    add_vector_kernel<<<n, S32_THREADS, 0, stream>>>(x, v, hidden);
     LLMS_LAUNCH_CHECK();
 }
 

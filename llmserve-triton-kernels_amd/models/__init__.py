@@ -1,3 +1,3 @@
 """Architectures: each module registers a name, a configuration class and a spec builder."""
 
-from . import dibepel, felavik, llama, milozen  # noqa: F401
+from . import dibepel, felavik, llama, milozen, nolavik  # noqa: F401

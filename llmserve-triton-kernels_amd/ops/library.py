@@ -1012,14 +1012,24 @@ def norm_store(q_out: torch.Tensor, proj: torch.Tensor, *, q_heads: int, k_heads
                q_norm: torch.Tensor | None = None, k_norm: torch.Tensor | None = None, eps: float = 0.0,
                temp_coef: float = 0.0, temp_every: int = 0, positions: torch.Tensor | None = None,
                slots: torch.Tensor | None = None, k_pool: torch.Tensor | None = None, v_pool: torch.Tensor | None = None,
-               block_size: int = 0) -> torch.Tensor:
-    """proj float32 [N, >= q_heads*dk + k_heads*dk + v_heads*dv] (q, k, v side by side; unit inner stride): every
+               block_size: int = 0, freq: torch.Tensor | None = None, unit_norm: bool = False) -> torch.Tensor:
+    """proj float32 [N, >= q_heads*dk + k_heads*dk + v_heads*dv] (q, k, v side by side; unit inner stride): with
+    `freq` (float32 [rot_dims / 2]) the first rot_dims numbers of every head of q and k are first turned by the
+    token's position (dimension i with dimension i + rot_dims / 2, angle position * freq[i]); `unit_norm`: every head
+    of q and k is divided by its root mean square with no weight; otherwise every
     head of q and of k is divided by its root mean square (eps inside the root) and multiplied by `q_norm` / `k_norm`
     (float32 [dk], shared by the heads; None: the head passes as it is); q is multiplied by
     1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) at position p (temp_every 0: no factor); rounded once: queries
     to q_out [N, q_heads*dk], keys and values to the tokens' cache slots (`slots`; None: nothing is stored)."""
-    dev = _dev(q_out, proj, q_norm, k_norm, positions, slots, k_pool, v_pool)
+    dev = _dev(q_out, proj, q_norm, k_norm, positions, slots, k_pool, v_pool, freq)
     n = proj.shape[0]
+    rot_dims = 0
+    if freq is not None:
+        _f32(freq, "freq")
+        rot_dims = 2 * freq.numel()
+        if rot_dims > dk:
+            raise ValueError(f"{rot_dims} turned dimensions in a head of {dk}")
+        _i32(positions, "positions", n)
     channels = (q_heads + k_heads) * dk + v_heads * dv
     if proj.dim() != 2 or proj.dtype != torch.float32 or proj.stride(1) != 1 or proj.shape[1] < channels:
         raise ValueError(f"proj must be float32 [N, >= {channels}] with unit inner stride")
@@ -1048,7 +1058,7 @@ def norm_store(q_out: torch.Tensor, proj: torch.Tensor, *, q_heads: int, k_heads
         c_int(_code(q_out)), _ptr(q_out), c_int(q_out.stride(0)), _ptr(proj), c_int(proj.stride(0)), _ptr(q_norm),
         _ptr(k_norm), c_float(eps), c_float(temp_coef), c_int(temp_every), _ptr(positions), _ptr(slots), _ptr(k_pool),
         _ptr(v_pool), c_int(n), c_int(q_heads), c_int(k_heads), c_int(dk), c_int(v_heads), c_int(dv), c_int(block_size),
-        _stream(dev)), "norm_store")
+        _ptr(freq), c_int(rot_dims), c_int(1 if unit_norm else 0), _stream(dev)), "norm_store")
     return q_out
 
 
@@ -1069,7 +1079,7 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
                     talk: torch.Tensor | None = None, lam: float = 0.0, head_norm: bool = False, eps: float = 0.0,
                     out_scale: float = 1.0, table_rows: torch.Tensor | None = None,
                     context_lens: torch.Tensor | None = None, dist_bias: torch.Tensor | None = None,
-                    gate: torch.Tensor | None = None) -> torch.Tensor:
+                    gate: torch.Tensor | None = None, sink: bool = False) -> torch.Tensor:
     """Attention of N new tokens over the paged cache, one workgroup per token (all its heads), float32 or bfloat16
     storage, 32-bit arithmetic.  q [N, heads*maps*dk] (head by head, a head's maps side by side); k_pool
     [pages, kv_heads*maps, block, dk]; v_pool [pages, kv_heads, dv, block]; out [N, heads*dv].  A query at
@@ -1079,7 +1089,8 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
     `head_norm`: each head's result is divided by its root mean square (eps inside the root) and multiplied by
     out_scale.  `context_lens` [B]: rows of a request of length 0 are padding and give zeros.  `dist_bias` float32
     [heads, R + 1]: dist_bias[h, min(i - j, R)] is added to the scores.  `gate` float32 [N, >= heads*dv] (unit inner
-    stride): the result is multiplied by sigmoid(gate)."""
+    stride): the result is multiplied by sigmoid(gate).  `sink`: the softmax's denominator holds one more term,
+    exp(0), a key of score zero without a value."""
     dev = _dev(out, q, k_pool, v_pool, block_tables, token_seq, positions, slopes, talk, table_rows, context_lens,
                dist_bias, gate)
     _check_dist_bias_and_gate(dist_bias, gate, heads, dv, q.shape[0])
@@ -1121,7 +1132,7 @@ def attend_composed(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tensor, v_
         c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
         c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), _ptr(dist_bias),
         c_int(dist_bias.shape[1] - 1 if dist_bias is not None else 0), _ptr(gate),
-        c_int(gate.stride(0) if gate is not None else 0), _stream(dev)),
+        c_int(gate.stride(0) if gate is not None else 0), c_int(1 if sink else 0), _stream(dev)),
         "attend_composed")
     return out
 
@@ -1308,6 +1319,12 @@ def streams_norm(out: torch.Tensor | None, x: torch.Tensor, weight: torch.Tensor
 # ------------------------------------------------------------------------------ attention through a latent
 
 
+def _pairing(pairing: str) -> int:
+    if pairing not in ("neighbours", "half"):
+        raise ValueError(f"pairing {pairing!r}; choose 'neighbours' (2i, 2i+1) or 'half' (i, i + dims/2)")
+    return 1 if pairing == "half" else 0
+
+
 def _latent_rotation(freq: torch.Tensor | None, dr: int) -> int:
     if freq is None:
         return 0
@@ -1320,10 +1337,12 @@ def _latent_rotation(freq: torch.Tensor | None, dr: int) -> int:
 
 def latent_prepare(z: torch.Tensor, *, col_q: int, q_rank: int, col_c: int | None, r: int, dr: int, wq: torch.Tensor,
                    wc: torch.Tensor | None, freq: torch.Tensor | None, positions: torch.Tensor, eps: float,
-                   cq: torch.Tensor, pool: torch.Tensor | None = None, slots: torch.Tensor | None = None) -> torch.Tensor:
+                   cq: torch.Tensor, pool: torch.Tensor | None = None, slots: torch.Tensor | None = None,
+                   pairing: str = "neighbours") -> torch.Tensor:
     """From the 32-bit input products z [N, columns]: cq [N, q_rank] = z[:, col_q:][:q_rank] over its root mean
     square times wq; with `col_c`, the cache rows pool[slots[n]] = [z_c over its root mean square times wc ; the dr
-    columns behind it with their first 2 len(freq) dimensions turned by the token's position (pairs 2i, 2i+1)].
+    columns behind it with their first 2 len(freq) dimensions turned by the token's position (pairs 2i, 2i+1; with
+    `pairing` "half" pairs i, i + len(freq))].
     pool [pages, 1, block, r + dr] in the dtype of cq."""
     dev = _dev(z, wq, wc, freq, positions, cq, pool, slots)
     if z.dim() != 2 or z.dtype != torch.float32 or z.stride(1) != 1:
@@ -1349,12 +1368,13 @@ def latent_prepare(z: torch.Tensor, *, col_q: int, q_rank: int, col_c: int | Non
     _check(load("latent").llms_latent_prepare(
         c_int(_code(cq)), _ptr(cq), _ptr(pool if col_c is not None else None), _ptr(z), c_int(z.stride(0)), c_int(col_q),
         c_int(q_rank), c_int(-1 if col_c is None else col_c), c_int(r), c_int(dr), _ptr(wq), _ptr(wc), _ptr(freq), c_int(dims),
-        _ptr(positions), _ptr(slots if col_c is not None else None), c_float(eps), c_int(n), _stream(dev)), "latent_prepare")
+        _ptr(positions), _ptr(slots if col_c is not None else None), c_float(eps), c_int(n), c_int(_pairing(pairing)),
+        _stream(dev)), "latent_prepare")
     return cq
 
 
 def latent_query(plain: torch.Tensor, folded: torch.Tensor, q: torch.Tensor, *, heads: int, dn: int, dr: int, r: int,
-                 freq: torch.Tensor | None, positions: torch.Tensor) -> None:
+                 freq: torch.Tensor | None, positions: torch.Tensor, pairing: str = "neighbours") -> None:
     """q [N, heads * (dn + dr)] float32 -> plain [N, heads * dn] (the unrotated parts) and folded[n, h, r:] (the
     rotated parts, turned); folded [N, heads * (r + dr)]."""
     dev = _dev(plain, folded, q, freq, positions)
@@ -1370,7 +1390,7 @@ def latent_query(plain: torch.Tensor, folded: torch.Tensor, q: torch.Tensor, *, 
         return
     _check(load("latent").llms_latent_query(
         c_int(_code(plain)), _ptr(plain), _ptr(folded), _ptr(q), c_int(heads), c_int(dn), c_int(dr), c_int(r), _ptr(freq),
-        c_int(dims), _ptr(positions), c_int(n), _stream(dev)), "latent_query")
+        c_int(dims), _ptr(positions), c_int(n), c_int(_pairing(pairing)), _stream(dev)), "latent_query")
 
 
 LATENT_ROW_MAX = 1024
@@ -1597,19 +1617,30 @@ MOE_MAX_TOP = 16
 
 def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_router: torch.Tensor, *,
                renormalize: bool = False, scores: str = "sigmoid", groups: int = 1, keep: int = 1,
-               renorm_eps: float = 0.0) -> None:
+               renorm_eps: float = 0.0, bias: torch.Tensor | None = None, extra_out: torch.Tensor | None = None) -> None:
     """Per row of h [N, hidden]: scores sigmoid(W_router h), or with `scores` "softmax" the softmax over all experts,
     in 32-bit; the `top` largest in descending order (the lower expert wins a tie) into chosen int32 [N, top], their
     scores (over their sum + `renorm_eps` with `renormalize`) into weight float32 [N, top].  `groups` > 1: the experts
     form that many equal groups of neighbours, a group's score is its largest, and only experts of the `keep` best
-    groups can be chosen."""
-    dev = _dev(chosen, weight, h, w_router)
+    groups can be chosen.  `bias` float32 [experts] is added to z.  `extra_out` float32 [N, extra]: w_router holds
+    `extra` more rows behind the experts', whose products with h are stored there as they are."""
+    dev = _dev(chosen, weight, h, w_router, bias, extra_out)
     _rows(h, "h")
     _rows(w_router, "w_router", h.shape[1])
     n, top = h.shape[0], chosen.shape[-1]
     _i32(chosen, "chosen", n * top)
     _f32(weight, "weight", n * top)
-    experts = w_router.shape[0]
+    extra = 0
+    if extra_out is not None:
+        if extra_out.dim() != 2 or extra_out.shape[0] != n:
+            raise ValueError("extra_out is [N, extra]")
+        extra = extra_out.shape[1]
+        _f32(extra_out, "extra_out", n * extra)
+    experts = w_router.shape[0] - extra
+    if experts < 1:
+        raise ValueError("w_router holds no experts' rows")
+    if bias is not None:
+        _f32(bias, "bias", experts)
     if h.dtype != w_router.dtype:
         raise ValueError("h and w_router differ in dtype")
     if not 1 <= top <= min(MOE_MAX_TOP, experts):
@@ -1623,7 +1654,7 @@ def moe_router(chosen: torch.Tensor, weight: torch.Tensor, h: torch.Tensor, w_ro
     _check(load("moe").llms_moe_router(
         c_int(_code(h)), _ptr(chosen), _ptr(weight), _ptr(h), _ptr(w_router), c_int(n), c_int(h.shape[1]), c_int(experts),
         c_int(top), c_int(1 if renormalize else 0), c_int(1 if scores == "softmax" else 0), c_int(groups), c_int(keep),
-        c_float(renorm_eps), _stream(dev)), "moe_router")
+        c_float(renorm_eps), _ptr(bias), c_int(extra), _ptr(extra_out), _stream(dev)), "moe_router")
 
 
 def moe_sort(chosen: torch.Tensor, experts: int):
@@ -1694,11 +1725,13 @@ def moe_scatter(xs: torch.Tensor, place: torch.Tensor, h: torch.Tensor, chosen: 
                                         _ptr(seg), c_int(pairs), c_int(h.shape[1]), c_int(top), _stream(dev)), "moe_scatter")
 
 
-def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weight: torch.Tensor | None = None) -> torch.Tensor:
+def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weight: torch.Tensor | None = None, *,
+                always: torch.Tensor | None = None, always_gate: torch.Tensor | None = None) -> torch.Tensor:
     """y[n] = sum_k rows[place[n, k]] in the order of k (times weight[n, k] where `weight`, float32 [N, top], is
     given); y float32 [N, hidden], rows float32 [pairs, hidden] or [parts, pairs, hidden] (partial sums of each row,
-    added in the order of the parts)."""
-    dev = _dev(y, rows, place, weight)
+    added in the order of the parts).  `always` float32 [N, hidden]: a result that every token adds last, times
+    sigmoid(always_gate[n]) where `always_gate` float32 [N] is given."""
+    dev = _dev(y, rows, place, weight, always, always_gate)
     n, hidden = y.shape
     _f32(y, "y")
     _f32(rows, "rows")
@@ -1710,10 +1743,17 @@ def moe_combine(y: torch.Tensor, rows: torch.Tensor, place: torch.Tensor, weight
         raise ValueError("rows has top rows of y's width per row of y")
     if weight is not None:
         _f32(weight, "weight", pairs)
+    if always is not None:
+        _f32(always, "always", n * hidden)
+    if always_gate is not None:
+        if always is None:
+            raise ValueError("always_gate comes with always")
+        _f32(always_gate, "always_gate", n)
     if n == 0:
         return y
     _check(load("moe").llms_moe_combine(_ptr(y), _ptr(rows), _ptr(place), c_int(n), c_int(hidden), c_int(top), c_int(parts),
-                                        c_long(pairs * hidden), _ptr(weight), _stream(dev)), "moe_combine")
+                                        c_long(pairs * hidden), _ptr(weight), _ptr(always), _ptr(always_gate), _stream(dev)),
+           "moe_combine")
     return y
 
 
@@ -1887,4 +1927,230 @@ def weighted_sum(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor, scale_a: f
     if out.numel():
         _check(load("stream32").llms_weighted_sum(_ptr(out), _ptr(a), _ptr(b), c_float(scale_a), c_float(scale_b),
                                                   ctypes.c_size_t(out.numel()), _stream(dev)), "weighted_sum")
+    return out
+
+
+# ------------------------------------------------------------------------------ a stream that sublayers join through a norm
+
+
+def normed_add_norm(out: torch.Tensor | None, x: torch.Tensor, weight: torch.Tensor | None, eps: float, *,
+                    y: torch.Tensor | None = None, y_weight: torch.Tensor | None = None, y_eps: float = 0.0,
+                    rows: torch.Tensor | None = None) -> torch.Tensor | None:
+    """x float32 [N, hidden], in one kernel: with `y` float32 [N, hidden], x += y / sqrt(mean(y^2) + y_eps) * y_weight
+    (stored into x unless `rows` picks rows); out = x / sqrt(mean(x^2) + eps) * weight, rounded once to out's dtype.
+    `rows` int32 [R]: out[r] comes from row rows[r] and nothing is stored.  `out` None: only the sum."""
+    dev = _dev(out, x, weight, y, y_weight, rows)
+    if x.dim() != 2 or x.dtype != torch.float32 or not x.is_contiguous():
+        raise ValueError(f"x must be a contiguous float32 [N, hidden] tensor, got {tuple(x.shape)} {x.dtype}")
+    n, hidden = x.shape
+    if hidden * 4 > 128 * 1024:
+        raise ValueError("rows of up to 32,768 elements")
+    if y is not None:
+        _f32(y, "y", n * hidden)
+        _f32(y_weight, "y_weight", hidden)
+    n_out = n
+    if rows is not None:
+        _i32(rows, "rows")
+        n_out = rows.numel()
+    if out is not None:
+        _rows(out, "out", hidden)
+        if out.shape[0] != n_out:
+            raise ValueError(f"out has {out.shape[0]} rows, expected {n_out}")
+        _f32(weight, "weight", hidden)
+    elif y is None or rows is not None:
+        raise ValueError("nothing to do: no output and nothing to store")
+    if n_out == 0:
+        return out
+    _check(load("stream32").llms_normed_add_norm(
+        c_int(_code(out) if out is not None else 0), _ptr(out), _ptr(x), _ptr(y), _ptr(y_weight), _ptr(weight), _ptr(rows),
+        c_int(n_out), c_int(hidden), c_float(y_eps), c_float(eps), c_int(1 if rows is None else 0), _stream(dev)),
+        "normed_add_norm")
+    return out
+
+
+def add_vector(x: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """x[..., :] += v for a contiguous float32 x whose last dimension is v's length."""
+    dev = _dev(x, v)
+    hidden = v.numel()
+    _f32(v, "v")
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.shape[-1] != hidden:
+        raise ValueError("x must be contiguous float32 with rows of v's length")
+    n = x.numel() // max(hidden, 1)
+    if n:
+        _check(load("stream32").llms_add_vector(_ptr(x), _ptr(v), c_int(n), c_int(hidden), _stream(dev)), "add_vector")
+    return x
+
+
+# ------------------------------------------------------------------------------ recurrences over a state of fixed size
+
+c_size_t = ctypes.c_size_t
+
+
+def _state_rows(state: torch.Tensor, state_slots: torch.Tensor, need: int, offset: int, what: str) -> int:
+    """state float32 [slots, numbers]: the stride between slots, after checking that [offset, offset + need) lies inside."""
+    if state.dim() != 2 or state.dtype != torch.float32 or not state.is_contiguous():
+        raise ValueError("state must be a contiguous float32 [slots, numbers] tensor")
+    if offset < 0 or offset + need > state.shape[1]:
+        raise ValueError(f"{what}: {need} numbers at {offset} do not fit a slot of {state.shape[1]}")
+    _i32(state_slots, "state_slots")
+    return state.shape[1]
+
+
+def _f32_matrix(t: torch.Tensor, name: str, rows: int, min_cols: int) -> None:
+    if t.dtype != torch.float32 or t.dim() != 2 or t.stride(1) != 1 or t.shape[0] != rows or t.shape[1] < min_cols:
+        raise ValueError(f"{name} must be float32 [{rows}, >= {min_cols}] with unit inner stride")
+
+
+def conv_act(u: torch.Tensor, u_col: int, channels: int, taps_w: torch.Tensor, *, bias: torch.Tensor | None = None,
+             state: torch.Tensor | None = None, ring_offset: int = 0, batch=None, out32: torch.Tensor | None = None,
+             out16: torch.Tensor | None = None, activation: str | None = "silu") -> None:
+    """A causal convolution per channel over time on columns u_col .. u_col + channels of u (float32 [N, >=]):
+    y_t = act(bias + sum_j taps_w[c, j] u_(t - taps + 1 + j)), zeros before the sequence; taps_w float32 [channels,
+    taps] with the last column for the present token.  A request's last taps - 1 rows are a ring [taps - 1, channels]
+    at `ring_offset` of its slot of `state` (float32 [slots, numbers]), indexed by position and brought up to date here.
+    The result goes to out32 (float32 [N, channels]) and/or out16 ([N, channels] in any kernel dtype).  `batch` brings
+    token_seq, positions, cu_seqlens, context_lens, state_slots, num_seqs and max_count."""
+    dev = _dev(u, taps_w, bias, state, out32, out16)
+    n = u.shape[0]
+    _f32_matrix(u, "u", n, u_col + channels)
+    taps = taps_w.shape[1]
+    _f32(taps_w, "taps_w", channels * taps)
+    if bias is not None:
+        _f32(bias, "bias", channels)
+    if activation not in (None, "silu"):
+        raise ValueError(f"activation {activation!r}")
+    slot_stride = 0
+    if taps > 1:
+        slot_stride = _state_rows(state, batch.state_slots, (taps - 1) * channels, ring_offset, "conv_act")
+    for t, name in ((out32, "out32"), (out16, "out16")):
+        if t is not None and (t.dim() != 2 or t.stride(1) != 1 or t.shape[0] != n or t.shape[1] != channels):
+            raise ValueError(f"{name} must be [N, {channels}] with unit inner stride")
+    if out32 is not None and out32.dtype != torch.float32:
+        raise ValueError("out32 is float32")
+    if out32 is None and out16 is None:
+        raise ValueError("nothing to store")
+    for t, name in ((batch.token_seq, "token_seq"), (batch.positions, "positions")):
+        _i32(t, name, n)
+    _i32(batch.cu_seqlens, "cu_seqlens")
+    _i32(batch.context_lens, "context_lens")
+    if n == 0:
+        return
+    lib = load("recurrent")
+    single = taps > 1 and batch.max_count == 1 and batch.num_seqs == n  # every request brings one token
+    _check(lib.llms_conv_act(
+        c_int(_code(out16) if out16 is not None else 0), _ptr(out32), c_int(out32.stride(0) if out32 is not None else 0),
+        _ptr(out16), c_int(out16.stride(0) if out16 is not None else 0), _ptr(u), c_int(u.stride(0)), c_int(u_col),
+        _ptr(taps_w), _ptr(bias), c_int(taps), c_int(channels), _ptr(state), c_size_t(slot_stride), c_size_t(ring_offset),
+        _ptr(batch.state_slots), _ptr(batch.token_seq), _ptr(batch.positions), _ptr(batch.cu_seqlens),
+        _ptr(batch.context_lens), c_int(n), c_int(1 if activation == "silu" else 0), c_int(1 if single else 0),
+        _stream(dev)), "conv_act")
+    if taps > 1 and not single:
+        _check(lib.llms_conv_ring(_ptr(state), c_size_t(slot_stride), c_size_t(ring_offset), _ptr(batch.state_slots), _ptr(u),
+                                  c_int(u.stride(0)), c_int(u_col), _ptr(batch.cu_seqlens), _ptr(batch.context_lens),
+                                  c_int(batch.num_seqs), c_int(taps), c_int(channels), _stream(dev)), "conv_ring")
+
+
+SCAN_MAX_STATES = 256
+
+
+def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: int, low: torch.Tensor, b_col: int, c_col: int,
+                   dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_neg: torch.Tensor, d_skip: torch.Tensor,
+                   state: torch.Tensor, scan_offset: int, batch) -> torch.Tensor:
+    """Per request, token by token, per channel c and state n:  S[c, n] <- exp(dt_c a_neg[c, n]) S[c, n] + dt_c x_c B_n,
+    y_c = sum_n S[c, n] C_n + d_skip[c] x_c, with dt = softplus(dt_raw + dt_bias); out[t, c] = y_c silu(z_c), rounded
+    once.  x float32 [N, channels]; z float32 [N, >= z_col + channels]; low float32 [N, >=] with B at b_col and C at
+    c_col (`states` numbers each); dt_raw float32 [N, channels]; S float32 [channels, states] at `scan_offset` of the
+    request's slot of `state`, read before the first token and left behind the last."""
+    dev = _dev(out, x, z, low, dt_raw, dt_bias, a_neg, d_skip, state)
+    n, channels = x.shape
+    if a_neg.dim() != 2 or a_neg.shape[0] != channels:
+        raise ValueError("a_neg is [channels, states]")
+    states = a_neg.shape[1]
+    if not 1 <= states <= SCAN_MAX_STATES:
+        raise ValueError(f"1 to {SCAN_MAX_STATES} states per channel, got {states}")
+    _f32_matrix(x, "x", n, channels)
+    _f32_matrix(z, "z", n, z_col + channels)
+    _f32_matrix(low, "low", n, max(b_col, c_col) + states)
+    _f32_matrix(dt_raw, "dt_raw", n, channels)
+    _f32(dt_bias, "dt_bias", channels)
+    _f32(a_neg, "a_neg", channels * states)
+    _f32(d_skip, "d_skip", channels)
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape != (n, channels):
+        raise ValueError(f"out must be [N, {channels}] with unit inner stride")
+    slot_stride = _state_rows(state, batch.state_slots, channels * states, scan_offset, "selective_scan")
+    _i32(batch.cu_seqlens, "cu_seqlens")
+    _i32(batch.context_lens, "context_lens")
+    if n == 0:
+        return out
+    _check(load("recurrent").llms_selective_scan(
+        c_int(_code(out)), _ptr(out), c_int(out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(z), c_int(z.stride(0)),
+        c_int(z_col), _ptr(low), c_int(low.stride(0)), c_int(b_col), c_int(c_col), _ptr(dt_raw), c_int(dt_raw.stride(0)),
+        _ptr(dt_bias), _ptr(a_neg), _ptr(d_skip), c_int(channels), c_int(states), _ptr(state), c_size_t(slot_stride),
+        c_size_t(scan_offset), _ptr(batch.state_slots), _ptr(batch.cu_seqlens), _ptr(batch.context_lens),
+        c_int(batch.num_seqs), _stream(dev)), "selective_scan")
+    return out
+
+
+def unit_heads(x: torch.Tensor, *, q_col: int, k_col: int, q_heads: int, k_heads: int, dk: int, eps: float,
+               q_factor: float = 1.0) -> torch.Tensor:
+    """In place on x (float32 [N, >=]): every head of dk numbers among the q_heads at q_col and the k_heads at k_col is
+    divided by sqrt(its sum of squares + eps); the q heads are also multiplied by q_factor."""
+    dev = _dev(x)
+    n = x.shape[0]
+    _f32_matrix(x, "x", n, max(q_col + q_heads * dk, k_col + k_heads * dk))
+    if n:
+        _check(load("recurrent").llms_unit_heads(_ptr(x), c_int(x.stride(0)), c_int(q_col), c_int(k_col), c_int(q_heads),
+                                                 c_int(k_heads), c_int(dk), c_float(eps), c_float(q_factor), c_int(n),
+                                                 _stream(dev)), "unit_heads")
+    return x
+
+
+DELTA_MAX_KEY = 256
+
+
+def delta_scan(o: torch.Tensor, qkv: torch.Tensor, *, q_col: int, k_col: int, v_col: int, gates: torch.Tensor, a_col: int,
+               b_col: int, a_log: torch.Tensor, dt_bias: torch.Tensor, heads: int, kv_heads: int, dk: int, dv: int,
+               state: torch.Tensor, scan_offset: int, batch) -> torch.Tensor:
+    """The gated delta rule per request, token by token, per head h over S [dk, dv] (q and k from head h / (heads /
+    kv_heads)):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with beta = sigmoid(gates[:, b_col + h])
+    and g = exp(-exp(a_log[h]) softplus(gates[:, a_col + h] + dt_bias[h])).  qkv float32 [N, >=] holds the prepared q
+    (kv_heads * dk at q_col), k (at k_col) and v (heads * dv at v_col); o float32 [N, heads * dv]; S float32 [heads, dk,
+    dv] at `scan_offset` of the request's slot of `state`."""
+    dev = _dev(o, qkv, gates, a_log, dt_bias, state)
+    n = qkv.shape[0]
+    if heads % kv_heads or not 1 <= dk <= DELTA_MAX_KEY:
+        raise ValueError(f"heads must be a multiple of kv_heads and keys hold 1 to {DELTA_MAX_KEY} numbers")
+    _f32_matrix(qkv, "qkv", n, max(q_col + kv_heads * dk, k_col + kv_heads * dk, v_col + heads * dv))
+    _f32_matrix(gates, "gates", n, max(a_col, b_col) + heads)
+    _f32_matrix(o, "o", n, heads * dv)
+    _f32(a_log, "a_log", heads)
+    _f32(dt_bias, "dt_bias", heads)
+    slot_stride = _state_rows(state, batch.state_slots, heads * dk * dv, scan_offset, "delta_scan")
+    _i32(batch.cu_seqlens, "cu_seqlens")
+    _i32(batch.context_lens, "context_lens")
+    if n == 0:
+        return o
+    _check(load("recurrent").llms_delta_scan(
+        _ptr(o), c_int(o.stride(0)), _ptr(qkv), c_int(qkv.stride(0)), c_int(q_col), c_int(k_col), c_int(v_col), _ptr(gates),
+        c_int(gates.stride(0)), c_int(a_col), c_int(b_col), _ptr(a_log), _ptr(dt_bias), c_int(heads), c_int(kv_heads),
+        c_int(dk), c_int(dv), _ptr(state), c_size_t(slot_stride), c_size_t(scan_offset), _ptr(batch.state_slots),
+        _ptr(batch.cu_seqlens), _ptr(batch.context_lens), c_int(batch.num_seqs), _stream(dev)), "delta_scan")
+    return o
+
+
+def delta_finish(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, gate_col: int, weight: torch.Tensor, *, heads: int,
+                 dv: int, eps: float) -> torch.Tensor:
+    """out[n, h] = o[n, h] / sqrt(mean(o[n, h]^2) + eps) * weight * silu(gate[n, gate_col + h dv ..]), rounded once;
+    o float32 [N, heads * dv], weight float32 [dv] shared by the heads, gate float32 [N, >=]."""
+    dev = _dev(out, o, gate, weight)
+    n = o.shape[0]
+    _f32_matrix(o, "o", n, heads * dv)
+    _f32_matrix(gate, "gate", n, gate_col + heads * dv)
+    _f32(weight, "weight", dv)
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape != (n, heads * dv):
+        raise ValueError(f"out must be [N, {heads * dv}] with unit inner stride")
+    if n:
+        _check(load("recurrent").llms_delta_finish(
+            c_int(_code(out)), _ptr(out), c_int(out.stride(0)), _ptr(o), c_int(o.stride(0)), _ptr(gate), c_int(gate.stride(0)),
+            c_int(gate_col), _ptr(weight), c_int(heads), c_int(dv), c_float(eps), c_int(n), _stream(dev)), "delta_finish")
     return out

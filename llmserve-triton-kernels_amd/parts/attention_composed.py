@@ -19,6 +19,12 @@ Parameters (a `PartSpec` of kind "composed_attention"):
   bias                  q, k and v have biases (tensors "<name>.b"), added in the projection
   qk_norm_eps           every head of q and of k is RMS-normed over its dk numbers with a weight of size dk that all
                         heads share (tensors "q.norm", "k.norm"; eps inside the root); None: no such norm
+  qk_norm_weight        False: that norm has no weight (and no tensors)
+  rotary                {base, dims, scaling}: before that norm the first `dims` numbers of every head of q and k are
+                        turned by the position, dimension i together with dimension i + dims / 2 by the angle
+                        p * f_i, f_i = base^(-2i / dims); `scaling` {factor, low, high, original} stretches long
+                        wavelengths (see `scaled_frequencies`); None: no rotation
+  sink                  the softmax's denominator holds one more term exp(0): a key of score zero without a value
   query_temperature     {coef, every}: q at position p is multiplied by 1 + coef ln(floor((p + 1) / every) + 1)
   distance_table        {rows: B, farthest: D}: a learned bias per head and distance, tensor "rel" [B, H], added to the
                         scaled score: rel[bucket(i - j), h] with bucket(n) = n for n < B/2 and
@@ -71,6 +77,25 @@ def bias_by_distance(table: torch.Tensor, farthest: int) -> torch.Tensor:
     return table.float()[index].t().contiguous()
 
 
+def scaled_frequencies(base: float, dims: int, scaling: dict | None = None) -> list[float]:
+    """f_i = base^(-2i / dims) for i < dims / 2.  With `scaling` {factor, low, high, original} a frequency whose
+    wavelength 2 pi / f lies below original / high stays, one beyond original / low is divided by factor, and between
+    the two it is (1 - s) f / factor + s f with s = (original / wavelength - low) / (high - low)."""
+    out = []
+    for i in range(dims // 2):
+        f = float(base) ** (-2.0 * i / dims)
+        if scaling:
+            factor, low, high, original = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+            wavelength = 2.0 * math.pi / f
+            if wavelength > original / low:
+                f = f / factor
+            elif wavelength >= original / high:
+                s = (original / wavelength - low) / (high - low)
+                f = (1.0 - s) * f / factor + s * f
+        out.append(f)
+    return out
+
+
 def _fill_rel(shape, generator, device, options):
     """A distance table: moderate biases."""
     return 0.5 * torch.randn(shape, generator=generator, dtype=torch.float32, device=device)
@@ -116,6 +141,13 @@ class ComposedAttention(Mixer):
         self.maps = 2 if self.differential else 1
         self.bias = bool(spec.get("bias", False))
         self.qk_norm_eps = spec.get("qk_norm_eps")
+        self.qk_norm_weight = bool(spec.get("qk_norm_weight", True))
+        rotary = spec.get("rotary") or None
+        self.rot_dims = int(rotary.get("dims", 0)) if rotary else 0
+        self.rot_freq = scaled_frequencies(float(rotary.get("base", 10000.0)), self.rot_dims, rotary.get("scaling")) \
+            if self.rot_dims else None
+        self.sink = bool(spec.get("sink", False))
+        self.freq = None
         temp = spec.get("query_temperature") or {}
         self.temp_coef, self.temp_every = float(temp.get("coef", 0.0)), int(temp.get("every", 0))
         table = spec.get("distance_table")
@@ -124,8 +156,12 @@ class ComposedAttention(Mixer):
         self.output_gate = bool(spec.get("output_gate", False))
         if table and (self.rel_rows < 2 or self.rel_farthest <= self.rel_rows // 2):
             raise ValueError("a distance table has at least 2 rows and reaches beyond the distances that have a row each")
-        if (self.qk_norm_eps is not None or self.temp_every) and self.taps > 0:
-            raise ValueError("normed or position-scaled queries do not go together with a convolution")
+        if (self.qk_norm_eps is not None or self.temp_every or self.rot_dims) and self.taps > 0:
+            raise ValueError("normed, turned or position-scaled queries do not go together with a convolution")
+        if self.rot_dims % 2 or not 0 <= self.rot_dims <= self.head_dim:
+            raise ValueError(f"rotary.dims={self.rot_dims} must be even and at most head_dim={self.head_dim}")
+        if self.rot_dims and self.differential:
+            raise ValueError("a rotation and two score maps per head do not go together")
         if self.temp_every < 0:
             raise ValueError("query_temperature.every must be positive")
         self.dist_bias = self.q_norm = self.k_norm = self.in_bias = None
@@ -188,7 +224,7 @@ class ComposedAttention(Mixer):
         if self.bias:
             for key, channels in (("q_bias", self.cq), ("k_bias", self.ck), ("v_bias", self.cv)):
                 infos[n[key]] = ParamInfo((channels,), "around_zero")
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_weight:
             infos[n["q_norm"]] = ParamInfo((self.head_dim,), "norm")
             infos[n["k_norm"]] = ParamInfo((self.head_dim,), "norm")
         if self.rel_rows:
@@ -208,7 +244,9 @@ class ComposedAttention(Mixer):
             if self.output_gate:
                 biases.append(torch.zeros(self.num_heads * self.value_dim, dtype=biases[0].dtype, device=dev))
             self.in_bias = torch.cat(biases).contiguous()
-        if self.qk_norm_eps is not None:
+        if self.rot_dims:
+            self.freq = torch.tensor(self.rot_freq, dtype=torch.float64).to(torch.float32).to(dev)
+        if self.qk_norm_eps is not None and self.qk_norm_weight:
             self.q_norm, self.k_norm = tensors[n["q_norm"]].float().contiguous(), tensors[n["k_norm"]].float().contiguous()
         if self.rel_rows:
             self.dist_bias = bias_by_distance(tensors[n["rel"]], self.rel_farthest)
@@ -243,12 +281,13 @@ class ComposedAttention(Mixer):
         proj = projected if projected is not None else linear(x, self.qkv_weight, self.in_bias, out_dtype=torch.float32)
         q = torch.empty((proj.shape[0], self.cq), dtype=x.dtype, device=x.device)
         gate = proj[:, self.cq + self.ck + self.cv:] if self.output_gate else None
-        if self.qk_norm_eps is not None or self.temp_every:
+        if self.qk_norm_eps is not None or self.temp_every or self.rot_dims:
             ops.norm_store(q, proj, q_heads=heads * self.maps, k_heads=kv * self.maps, dk=dk, v_heads=kv, dv=dv,
                            q_norm=self.q_norm, k_norm=self.k_norm, eps=float(self.qk_norm_eps or 0.0),
                            temp_coef=self.temp_coef, temp_every=self.temp_every, positions=batch.positions,
                            slots=view.slots if paged.store else None, k_pool=paged.k_pool, v_pool=paged.v_pool,
-                           block_size=paged.block_size)
+                           block_size=paged.block_size, freq=self.freq,
+                           unit_norm=self.qk_norm_eps is not None and not self.qk_norm_weight)
             out = torch.empty((proj.shape[0], heads * dv), dtype=x.dtype, device=x.device)
             self.attend(out, q, paged, view, batch, gate)
             return linear(out, self.o_weight, out_dtype=self.result_dtype)
@@ -278,11 +317,12 @@ class ComposedAttention(Mixer):
                       keep_first=self.keep_first, chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk,
                       lam=self.lam, head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
                       out_scale=self.head_norm_scale, table_rows=batch.state_slots)
-        if (gate is not None and (self.talking or gate.data_ptr() % 16 or gate.stride(0) % 4)) or \
+        if self.sink or (gate is not None and (self.talking or gate.data_ptr() % 16 or gate.stride(0) % 4)) or \
                 not ops.attend_composed_mfma_supported(
                 q.dtype, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, paged.block_size, self.talking):
             ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
-                                context_lens=batch.context_lens, dist_bias=self.dist_bias, gate=gate, **common)
+                                context_lens=batch.context_lens, dist_bias=self.dist_bias, gate=gate, sink=self.sink,
+                                **common)
             return
         args = (out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
         common.update(dist_bias=self.dist_bias, gate=gate)

@@ -8,6 +8,8 @@ Parameters (a `PartSpec` of kind "latent_attention"):
                        None: everything); default: window
   rotary_base, rotary_dims   pairs (2i, 2i+1) of the first rotary_dims numbers of a rotated part are turned by
                        position * base^(-2i / rotary_dims); the rest of the part passes
+  rotary_pairing       "neighbours" (default) or "half": dimension i turns together with dimension i + rotary_dims / 2
+  rotary_frequencies   the rotary_dims / 2 frequencies themselves, where they are not base^(-2i / rotary_dims)
   eps                  of the two latents' RMS norms (plain weights)
   own_latent           False: the layer has no key/value projection and reads another layer's cache rows
   output_gate          the heads' results are multiplied by sigmoid(W_g h) before the output projection
@@ -52,6 +54,10 @@ class LatentAttention(Mixer):
         self.cache_window = spec.get("cache_window", self.window)
         self.base = float(spec.get("rotary_base", 10000.0))
         self.dims = int(spec.get("rotary_dims", self.dr))
+        self.pairing = spec.get("rotary_pairing", "neighbours")
+        self.frequencies = spec.get("rotary_frequencies")
+        if self.frequencies is not None and 2 * len(self.frequencies) != self.dims:
+            raise ValueError("rotary_frequencies holds a frequency per turned pair")
         self.eps = float(spec["eps"])
         self.own_latent = bool(spec.get("own_latent", True))
         self.output_gate = bool(spec.get("output_gate", True))
@@ -107,7 +113,9 @@ class LatentAttention(Mixer):
         self.w_o = tensors[n["o"]].contiguous()
         self.wq_norm = tensors[n["dq_norm"]].float().contiguous()
         self.wc_norm = tensors[n["dkv_norm"]].float().contiguous() if self.own_latent else None
-        if self.dims:
+        if self.dims and self.frequencies is not None:
+            self.freq = torch.tensor([float(f) for f in self.frequencies], dtype=torch.float64).to(torch.float32).to(self.w_o.device)
+        elif self.dims:
             exponent = torch.arange(0, self.dims, 2, dtype=torch.float64) / self.dims
             self.freq = (1.0 / (self.base ** exponent)).to(torch.float32).to(self.w_o.device)
 
@@ -122,11 +130,13 @@ class LatentAttention(Mixer):
         cq = torch.empty((rows, self.q_rank), dtype=dtype, device=dev)
         ops.latent_prepare(z, col_q=0, q_rank=self.q_rank, col_c=self.col_c, r=r, dr=dr, wq=self.wq_norm, wc=self.wc_norm,
                            freq=self.freq, positions=batch.positions, eps=self.eps, cq=cq,
-                           pool=cache.k_pool if self.own_latent else None, slots=view.slots if self.own_latent else None)
+                           pool=cache.k_pool if self.own_latent else None, slots=view.slots if self.own_latent else None,
+                           pairing=self.pairing)
         q = linear(cq, self.w_uq, out_dtype=torch.float32)
         plain = torch.empty((rows, heads * dn), dtype=dtype, device=dev)
         folded = torch.empty((rows, heads * (r + dr)), dtype=dtype, device=dev)
-        ops.latent_query(plain, folded, q, heads=heads, dn=dn, dr=dr, r=r, freq=self.freq, positions=batch.positions)
+        ops.latent_query(plain, folded, q, heads=heads, dn=dn, dr=dr, r=r, freq=self.freq, positions=batch.positions,
+                         pairing=self.pairing)
         ops.grouped_product(folded.view(rows, heads, r + dr)[:, :, :r], plain.view(rows, heads, dn), self.w_absorb)
         mixed = torch.empty((rows, heads * r), dtype=dtype, device=dev)
         self.attend(mixed, folded, cache, view, batch)

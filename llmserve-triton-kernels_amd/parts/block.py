@@ -11,6 +11,10 @@ applies the gates and sums.
 where read and write are the sublayer's `Connection` (kind "residual": read is x itself and write adds; kind "hyper":
 weighted sums over the copies).  Each write is left open and done by the kernel that reads the streams next.
 
+"sandwich" is "streams" with a norm behind every sublayer as well as before it, over one stream:
+    x <- x + post_1(mixer(norm1(x)));  x <- x + post_2(feed_forward(norm2(x)))
+The sum through the second norm is left open (`NormedSum`) and done by the kernel that norms the stream next.
+
 "prenorm" is the reference's decoder layer (src/llmserve/model/llama.py:131-135):
     x = x + mixer(norm1(x));  x = x + feed_forward(norm2(x))
 The hidden state travels as (x, delta) with the last sum still open, so each residual
@@ -23,7 +27,7 @@ import torch
 
 from ..ops import library as ops
 from .linear import linear
-from .registry import ADDED_IN_PLACE, Block, DeferredNorm, GatedSum, OpenStreams, register_block
+from .registry import ADDED_IN_PLACE, Block, DeferredNorm, GatedSum, NormedSum, OpenStreams, register_block
 
 
 @register_block("prenorm")
@@ -144,3 +148,30 @@ class StreamsBlock(Block):
     @staticmethod
     def _result(y):
         return y if y.dtype == torch.float32 else y.float()
+
+
+@register_block("sandwich")
+class SandwichBlock(StreamsBlock):
+    """Norms before and behind each sublayer over one 32-bit stream: the roles of "streams" and, of the family "norm",
+    `mixer_post_norm` and `feed_forward_post_norm` (RMS norms with a weight: parts that offer `weight` and `eps`).  The
+    connections are plain ("residual"); the norms before the sublayers must close a `NormedSum`."""
+
+    ROLES = dict(StreamsBlock.ROLES, mixer_post_norm="norm", feed_forward_post_norm="norm")
+
+    def _read(self, norm, connection, x, delta):
+        if not getattr(norm, "closes_normed_sums", False):
+            raise ValueError(f"{type(norm).__name__} cannot close a sum through a norm")
+        if connection.streams != 1 or connection.read is not None:
+            raise ValueError("the sandwich arrangement keeps one plain stream")
+        return super()._read(norm, connection, x, delta)
+
+    def _joined(self, y, post):
+        return NormedSum(self._result(y), post.weight, post.eps)
+
+    def forward(self, x, delta, batch, cache):
+        h, x = self._read(self.mixer_norm, self.mixer_connection, x, delta)
+        delta = self._joined(self.mixer.forward(h, batch, cache), self.mixer_post_norm)
+        if getattr(self.feed_forward, "absent", False):
+            return x, delta
+        h, x = self._read(self.feed_forward_norm, self.feed_forward_connection, x, delta)
+        return x, self._joined(self.feed_forward.forward(h), self.feed_forward_post_norm)

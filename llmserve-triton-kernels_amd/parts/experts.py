@@ -6,7 +6,10 @@ pattern of an expert's matrices, default "e{e}.gate", "e{e}.up", "e{e}.down"), a
 out: scores ("sigmoid" or "softmax" over all experts), groups and keep (the experts form `groups` equal groups of
 neighbours, a group's score is its largest, only experts of the `keep` best groups can be chosen), renorm_eps (added
 to the sum that `renormalize` divides by), weight_on ("input": the weight multiplies the expert's input; "output":
-its result), unit ("clamped" or "silu").
+its result), unit ("clamped" or "silu"), router_bias (True: a bias per expert, tensor "<router>.b", is added to z),
+shared ({"intermediate": I, "gate": True or False}: one more SiLU-gated unit of its own width that every token uses,
+tensors "shared.gate", "shared.up", "shared.down"; with "gate" its result is multiplied by sigmoid(w_sg . h), one number
+per token, tensor "shared.sg" [1, hidden]).
 
 Router: z = W_router h in 32-bit, scores sigmoid(z) or softmax(z), the `top` largest chosen.  With weight_on
 "input" y = sum over chosen e of expert_e(w_e h), with "output" y = sum of w_e expert_e(h).  Expert, unit "clamped":
@@ -25,10 +28,12 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
+from .linear import linear
 from .registry import FeedForward, register_feed_forward
 from .spec import ParamInfo
 
-_DEFAULT_NAMES = {"router": "router", "gate": "e{e}.gate", "up": "e{e}.up", "down": "e{e}.down"}
+_DEFAULT_NAMES = {"router": "router", "gate": "e{e}.gate", "up": "e{e}.up", "down": "e{e}.down", "router_bias": "router.b",
+                  "shared_gate": "shared.gate", "shared_up": "shared.up", "shared_down": "shared.down", "shared_sg": "shared.sg"}
 
 
 @register_feed_forward("experts")
@@ -57,6 +62,13 @@ class Experts(FeedForward):
             raise ValueError(f"{self.groups} groups of which {self.keep} are kept do not fit {self.experts} experts "
                              f"of which {self.top} are chosen")
         self.names = dict(_DEFAULT_NAMES, **(spec.get("names") or {}))
+        self.router_bias = bool(spec.get("router_bias", False))
+        shared = spec.get("shared") or None
+        self.shared_intermediate = int(shared["intermediate"]) if shared else 0
+        self.shared_gated = bool(shared.get("gate", False)) if shared else False
+        if shared and self.shared_intermediate < 1:
+            raise ValueError("the shared unit needs a positive width")
+        self.w_shared_gate_up = self.w_shared_down = self.b_router = None
         if not 1 <= self.top <= min(self.experts, ops.MOE_MAX_TOP):
             raise ValueError(f"top={self.top} of {self.experts} experts (at most {ops.MOE_MAX_TOP})")
         self.w_router = self.w_gate_up = self.w_down = None
@@ -71,11 +83,26 @@ class Experts(FeedForward):
             infos[n["gate"].format(e=e)] = ParamInfo((i, h))
             infos[n["up"].format(e=e)] = ParamInfo((i, h))
             infos[n["down"].format(e=e)] = ParamInfo((h, i))
+        if self.router_bias:
+            infos[n["router_bias"]] = ParamInfo((self.experts,), "around_zero")
+        if self.shared_intermediate:
+            s = self.shared_intermediate
+            infos[n["shared_gate"]], infos[n["shared_up"]] = ParamInfo((s, h)), ParamInfo((s, h))
+            infos[n["shared_down"]] = ParamInfo((h, s))
+            if self.shared_gated:
+                infos[n["shared_sg"]] = ParamInfo((1, h))
         return infos
 
     def load(self, tensors):
         n = self.names
         self.w_router = tensors[n["router"]].contiguous()
+        if self.router_bias:
+            self.b_router = tensors[n["router_bias"]].float().contiguous()
+        if self.shared_intermediate:
+            self.w_shared_gate_up = torch.cat([tensors[n["shared_gate"]], tensors[n["shared_up"]]], dim=0).contiguous()
+            self.w_shared_down = tensors[n["shared_down"]].contiguous()
+            if self.shared_gated:  # the gate's row lies behind the experts' in the router's matrix: one kernel forms both
+                self.w_router = torch.cat([self.w_router, tensors[n["shared_sg"]].reshape(1, self.hidden)], dim=0).contiguous()
         # [E, 64 ceil(I / 32), H]: blocks of 32 gate rows and the 32 up rows of the same units, so that a thread of
         # the product holds both of a unit
         self.w_gate_up = ops.stack_paired(torch.stack([tensors[n["gate"].format(e=e)] for e in range(self.experts)]),
@@ -87,8 +114,15 @@ class Experts(FeedForward):
         pairs = rows * self.top
         chosen = torch.empty((rows, self.top), dtype=torch.int32, device=dev)
         weight = torch.empty((rows, self.top), dtype=torch.float32, device=dev)
+        shared_gate = torch.empty((rows, 1), dtype=torch.float32, device=dev) if self.shared_gated else None
         ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize, scores=self.scores,
-                       groups=self.groups, keep=self.keep, renorm_eps=self.renorm_eps)
+                       groups=self.groups, keep=self.keep, renorm_eps=self.renorm_eps, bias=self.b_router,
+                       extra_out=shared_gate)
+        shared = None
+        if self.shared_intermediate:
+            unit = torch.empty((rows, self.shared_intermediate), dtype=x.dtype, device=dev)
+            ops.silu_mul(unit, linear(x, self.w_shared_gate_up))
+            shared = linear(unit, self.w_shared_down, out_dtype=torch.float32)
         on_input = self.weight_on == "input"
         sorted_in = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
         place = torch.empty(pairs, dtype=torch.int32, device=dev)
@@ -106,4 +140,5 @@ class Experts(FeedForward):
         results = torch.empty(shape, dtype=torch.float32, device=dev)
         ops.grouped_product(results, act, self.w_down, segments=(seg, tiles), k_parts=parts)
         return ops.moe_combine(torch.empty((rows, self.hidden), dtype=torch.float32, device=dev), results, place,
-                               None if on_input else weight)
+                               None if on_input else weight, always=shared,
+                               always_gate=None if shared_gate is None else shared_gate.view(rows))

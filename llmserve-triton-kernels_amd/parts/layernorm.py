@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .registry import Norm, OpenStreams, register_norm
+from .registry import Norm, NormedSum, OpenStreams, register_norm
 from .spec import ParamInfo
 
 
@@ -79,6 +79,29 @@ class RMSNormStreams(LayerNorm32):
     rounded once.  Parameters as above."""
 
     center = False
+    closes_normed_sums = True  # `read_streams`, `add_norm` and `norm_rows` also take a `NormedSum` in the place of delta
+
+    def _one_stream(self, x):
+        x = self._streams(x)
+        if x.shape[1] != 1:
+            raise ValueError("a sum through a norm joins a stream of one copy")
+        return x.view(x.shape[0], self.hidden)
+
+    def read_streams(self, x, delta, connection=None, source=None):
+        if not isinstance(delta, NormedSum):
+            return super().read_streams(x, delta, connection, source)
+        if source is not None or (connection is not None and connection.read is not None):
+            raise ValueError("a sum through a norm joins one plain stream")
+        rows = self._one_stream(x)
+        out = torch.empty((rows.shape[0], self.hidden), dtype=self.ctx.dtype, device=x.device)
+        return ops.normed_add_norm(out, rows, self.weight, self.eps, y=delta.y, y_weight=delta.weight, y_eps=delta.eps)
+
+    def norm_rows(self, x, delta, rows):
+        if not isinstance(delta, NormedSum):
+            return super().norm_rows(x, delta, rows)
+        out = torch.empty((rows.numel(), self.hidden), dtype=self.ctx.dtype, device=x.device)
+        return ops.normed_add_norm(out, self._one_stream(x), self.weight, self.eps, y=delta.y, y_weight=delta.weight,
+                                   y_eps=delta.eps, rows=rows)
 
 
 @register_norm("none")

@@ -11,9 +11,11 @@ from __future__ import annotations
 
 import torch
 
-from . import (attention, attention_composed, attention_latent, block, connection, decay_attention, embedding,  # noqa: F401
-               experts, gate, layernorm, rmsnorm, rope, side_by_side, swiglu)  # (register the built-in parts)
-from .registry import BLOCKS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm, Part
+from ..ops import library as ops
+from . import (attention, attention_composed, attention_latent, block, connection, decay_attention, delta_rule, embedding,  # noqa: F401
+               experts, gate, layernorm, rmsnorm, rope, selective_scan, side_by_side, swiglu)  # (register the built-in parts)
+from .registry import (BLOCKS, CONNECTIONS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, BuildContext, DeferredNorm,
+                       OpenStreams, Part)
 from .spec import ModelSpec, ParamInfo
 
 
@@ -27,6 +29,8 @@ class Model:
         self.head = HEADS.build(spec.head, ctx)
         self.blocks = []
         self._sources = None
+        self._shift_rows = {pos: row for pos, row in spec.shifts}
+        self.shift_table = None  # float32 [rows, hidden] on the device
         families = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "gate": GATES,
                     "connection": CONNECTIONS}
         for index, layer in enumerate(spec.layers):
@@ -52,6 +56,8 @@ class Model:
         for prefix, part in self._parts():
             for local, info in part.param_infos().items():
                 infos[prefix + local] = info
+        if self._shift_rows:
+            infos[self.spec.weights["shifts"]] = ParamInfo((max(self._shift_rows.values()) + 1, self.spec.hidden_size), "around_zero")
         return infos
 
     def load(self, tensors: dict[str, torch.Tensor]) -> None:
@@ -62,6 +68,8 @@ class Model:
             part.load({local: tensors[prefix + local] for local in part.param_infos()})
         if getattr(self.head, "tied", False):
             self.head.load({"weight": self.embedding.weight})
+        if self._shift_rows:
+            self.shift_table = tensors[self.spec.weights["shifts"]].float().contiguous()
 
     def libraries(self, dtype_name: str) -> tuple[str, ...]:
         """Kernel libraries the model's parts name, in first-use order without repeats."""
@@ -69,6 +77,8 @@ class Model:
         for _, part in self._parts():
             for name in part.libraries(dtype_name):
                 names[name] = None
+        if self._shift_rows:
+            names["stream32"] = None
         return tuple(names)
 
     def graph_safe(self) -> bool:
@@ -99,6 +109,15 @@ class Model:
                 sources.append(max(p for p in range(pos) if self.spec.schedule[p] == src))
         return sources
 
+    def _shift(self, x, delta, row: int) -> None:
+        """hidden state += shift_table[row] for every token.  The hidden state is x + (the open sum delta); where that
+        sum does not depend on x, adding to x now is adding behind it."""
+        if x.dtype != torch.float32:
+            raise ValueError("shifts are added to a 32-bit residual stream")
+        if isinstance(delta, OpenStreams) and delta.connection.mix is not None:
+            raise ValueError("a shift behind a write that mixes the streams is not supported")
+        ops.add_vector(x, self.shift_table[row])
+
     # ---- one step ----------------------------------------------------------------------------
     def forward(self, batch, storage) -> torch.Tensor:
         """Logits [R, vocab] in 32-bit at `batch.logit_rows` (empty tensor when R = 0)."""
@@ -111,6 +130,8 @@ class Model:
             self._sources = self.cache_sources()
         for pos, index in enumerate(self.spec.schedule):
             cache = storage.layer_cache(pos, self._sources[pos])
+            if pos in self._shift_rows:
+                self._shift(x, delta, self._shift_rows[pos])
             x, delta = self.blocks[index].forward(x, delta, batch, cache)
         rows = batch.logit_rows
         if rows.numel() == 0:

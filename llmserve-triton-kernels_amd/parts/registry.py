@@ -122,6 +122,17 @@ class OpenStreams:
     connection: "Connection"
 
 
+@dataclass
+class NormedSum:
+    """A residual sum that is still open: x += y / sqrt(mean(y^2) + eps) * weight, a sublayer's result y (32-bit) joining
+    a 32-bit stream through an RMS norm of its own.  It travels in the place of `delta`; a norm that sets
+    `closes_normed_sums` does the sum in the kernel that norms the stream for the next sublayer."""
+
+    y: torch.Tensor
+    weight: torch.Tensor
+    eps: float
+
+
 def as_tensor(delta):
     """`delta` as a tensor in the model's dtype (None stays None)."""
     return delta.total() if isinstance(delta, PartialSums) else delta

@@ -61,6 +61,9 @@ class ModelSpec:
     head: PartSpec
     weights: Mapping[str, str]  # roles "embedding", "final_norm", "head" -> checkpoint prefix
     unused_tensors: tuple[str, ...] = ()  # names a checkpoint may hold without the model reading them
+    # (entry of the schedule, row): before that entry runs, row `row` of the tensor named by weights["shifts"]
+    # ([rows, hidden]) is added to the hidden state of every token
+    shifts: tuple[tuple[int, int], ...] = ()
 
     def validate(self) -> None:
         n = len(self.layers)
@@ -69,6 +72,11 @@ class ModelSpec:
         for i in self.schedule:
             if not 0 <= i < n:
                 raise ValueError(f"schedule names layer {i}, but there are {n} layers")
+        if self.shifts and "shifts" not in self.weights:
+            raise ValueError("shifts need the name of their tensor (weights['shifts'])")
+        for pos, row in self.shifts:
+            if not 0 <= pos < len(self.schedule) or row < 0:
+                raise ValueError(f"shift ({pos}, {row}) names no entry of the schedule or no row")
         for i, layer in enumerate(self.layers):
             src = layer.cache_from
             if src is not None:
