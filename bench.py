@@ -26,10 +26,12 @@ first token, inter-token latency percentiles and the number of preemptions besid
 `--pages-fraction` shrinks the cache pool below what the whole workload needs, so that
 requests wait and are preempted.
 
-    python bench.py --workload designs [--design dibepel|milozen|felavik] [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
+    python bench.py --workload designs [--design dibepel|milozen|felavik|nolavik] [--beside llama|felavik|...] [--sizes 1b,7b] [--layers 6] [--batches 8,32] [--context 512]
 
 puts the Dibepel design (or, with `--design milozen`, the Milozen design: latent attention, experts, two streams; with
-`--design felavik`, the Felavik design: linear attention with a decay per head, gated softmax attention, experts in groups)
+`--design felavik`, the Felavik design: linear attention with a decay per head, gated softmax attention, experts in groups;
+with `--design nolavik`, the Nolavik design: latent attention, the gated delta rule, sink attention beside a selective scan,
+experts with a shared expert, a looped layer)
 beside the Llama decoder at equal layer sizes (width, heads, key/value heads, head size,
 feed-forward, vocabulary, layers; random weights): prefill tokens a second for one prompt of 2,048 tokens in one
 step, and decoded tokens a second at the given batch sizes behind `--context` tokens, both through the step
@@ -269,6 +271,31 @@ def felavik_config(size: dict, layers: int, experts: int = 8, top: int = 2) -> d
             "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "layers": entries}
 
 
+def nolavik_config(size: dict, layers: int, experts: int = 8, top: int = 2) -> dict:
+    """`layers` layer runs: latent attention (as many heads as the Llama shape, the head size unrotated and half of it
+    rotated, a latent of four head sizes), the gated delta rule (as many value heads, half as many query/key heads, 4 taps),
+    softmax attention with a sink of the Llama shape's heads and key/value heads (half of every head turned, stretched
+    frequencies) beside a selective scan as wide as the model (16 states a channel), in turn; the second layer runs twice
+    (the loop); every layer chooses `top` of `experts` experts of a quarter of the dense width and has a shared expert of
+    half of it (the active weights of the dense feed-forward)."""
+    dim, heads, width = size["dim"], size["heads"], size["width"]
+    mlp = {"kind": "moe", "expert": {"ff": size["ff"] // 4}, "router": {"experts": experts, "top": top},
+           "shared": {"ff": size["ff"] // 2}}
+    kinds = {
+        "latent_attention": {"heads": heads, "dim": dim, "rot_dim": dim // 2, "vdim": dim, "q_rank": 3 * width // 8,
+                             "kv_rank": 4 * dim, "scale": (dim + dim // 2) ** -0.5, "rot": {"base": 10000.0, "dims": dim // 2}},
+        "delta": {"heads": heads, "kv_heads": max(1, heads // 2), "dim": dim, "vdim": dim, "conv": 4},
+        "parallel": {"left": {"heads": heads, "kv_heads": size["kv_heads"], "dim": dim, "vdim": dim, "scale": 8.0 / dim,
+                              "rot": {"base": 500000.0, "dims": dim // 2,
+                                      "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+                     "right": {"inner": width, "state": 16, "dt_rank": width // 16, "conv": 4},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    order = ["latent_attention", "delta", "parallel"]
+    entries = [{"type": order[i % 3], "mixer": kinds[order[i % 3]], "mlp": mlp} for i in range(max(2, layers - 1))]
+    return {"architecture": "Nolavik", "vocab": size["vocab"], "width": width, "norm": {"eps": 1e-6}, "layers": entries,
+            "loop": {"start": 1, "stop": 2, "times": 2 if layers > 2 else 1}}
+
+
 def llama_config(size: dict, layers: int, positions: int) -> dict:
     return dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=size["vocab"], hidden_size=size["width"],
                 intermediate_size=size["ff"], num_hidden_layers=layers, num_attention_heads=size["heads"],
@@ -343,18 +370,21 @@ def designs(args) -> int:
 
     table = {}
     design = args.design
-    make = {"dibepel": dibepel_config, "milozen": milozen_config, "felavik": felavik_config}[design]
+    makers = {"dibepel": dibepel_config, "milozen": milozen_config, "felavik": felavik_config, "nolavik": nolavik_config}
+    make, beside = makers[design], args.beside
+    if beside == design:
+        raise SystemExit("--beside names the design itself")
     for name in [s for s in args.sizes.split(",") if s]:
         size = DESIGN_SIZES[name]
         layers = args.layers or 6
-        row = {"layers": layers, **size, design: measure(make(size, layers)),
-               "llama": measure(llama_config(size, layers, longest))}
-        row[f"{design}_over_llama"] = {k: round(row[design][k] / row["llama"][k], 3) for k in row[design]
-                                       if k.endswith("tok_s")}
+        other = llama_config(size, layers, longest) if beside == "llama" else makers[beside](size, layers)
+        row = {"layers": layers, **size, design: measure(make(size, layers)), beside: measure(other)}
+        row[f"{design}_over_{beside}"] = {k: round(row[design][k] / row[beside][k], 3) for k in row[design]
+                                          if k.endswith("tok_s")}
         table[name] = row
     first = table[next(iter(table))]
     title = design.capitalize()
-    line = {"metric": f"{title} beside Llama at equal layer sizes: decode tok/s (value: {title}, first size and batch), prefill tok/s",
+    line = {"metric": f"{title} beside {beside.capitalize()} at equal layer sizes: decode tok/s (value: {title}, first size and batch), prefill tok/s",
             "value": first[design][f"decode_b{batches[0]}_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps,
             "warmup": warmup, "ms_per_step": first[design][f"decode_b{batches[0]}_ms"], "higher_is_better": True,
             "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
@@ -485,7 +515,10 @@ def main() -> int:
                     help="run one phase only (for profiles; the line then holds zeros for the other); gemv: the "
                          "decode products alone, each over copies of its weight that do not fit the caches")
     ap.add_argument("--workload", choices=["steps", "serve", "designs"], default="steps")
-    ap.add_argument("--design", choices=["dibepel", "milozen", "felavik"], default="dibepel", help="designs: which design stands beside Llama")
+    ap.add_argument("--design", choices=["dibepel", "milozen", "felavik", "nolavik"], default="dibepel",
+                    help="designs: which design is measured")
+    ap.add_argument("--beside", choices=["llama", "dibepel", "milozen", "felavik", "nolavik"], default="llama",
+                    help="designs: the model it stands beside, at equal layer sizes")
     ap.add_argument("--sizes", default="1b,7b", help="designs: layer sizes to compare at")
     ap.add_argument("--batches", default="8,32", help="designs: decode batch sizes")
     ap.add_argument("--requests", type=int, default=64)

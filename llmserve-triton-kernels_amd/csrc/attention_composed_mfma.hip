@@ -67,6 +67,7 @@ struct MfmaArgs {
     float* ws_o;
     float scale, lambda, eps, out_scale;
     int head_norm;
+    int sink;  // the softmax's denominator holds one more term, exp(0) (without mixed heads)
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }  // v_exp_f32; 0 for -inf
@@ -345,6 +346,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
     };
 
     float col_l[MAXU][MAPS];  // a column's whole sum, once it is known
+    float col_m[MAXU][MAPS];  // and the reference its weights were taken against (for the sink's term)
     if constexpr (!TALK) {
         for (int round = 0; round < n_rounds; ++round) {
             const int group = (round * NS + slice) * NSG + share;
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
 #pragma unroll
         for (int uu = 0; uu < MAXU; ++uu)
 #pragma unroll
-            for (int m = 0; m < MAPS; ++m) col_l[uu][m] = column_sum(run_l[uu][m]);
+            for (int m = 0; m < MAPS; ++m) col_l[uu][m] = column_sum(run_l[uu][m]), col_m[uu][m] = run_m[uu][m];
         if (NS > 1) {  // the slices of a unit meet in LDS: [unit wave][slice][map]{m[16], l[16], o[dv][16]}
             const int per = 16 * (2 + dv);
 #pragma unroll
@@ -417,6 +419,7 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
                                 for (int r = 0; r < 4; ++r) acc_o[uu][m][t][r] += f * at[32 + (16 * t + 4 * q4 + r) * 16 + col];
                     }
                     col_l[uu][m] = total;
+                    col_m[uu][m] = top;
                 }
         }
     } else {
@@ -566,7 +569,14 @@ __global__ __launch_bounds__(THREADS) void attend_mfma_kernel(const MfmaArgs a) 
         if (!mine[uu]) continue;
         float mul[MAPS];
 #pragma unroll
-        for (int m = 0; m < MAPS; ++m) mul[m] = TALK ? 1.f : 1.f / col_l[uu][m];
+        for (int m = 0; m < MAPS; ++m) {
+            if constexpr (TALK) {
+                mul[m] = 1.f;
+            } else {  // (scores are in units of log2: the sink's score 0 stays 0)
+                const float l = a.sink ? col_l[uu][m] + fast_exp2(-col_m[uu][m]) : col_l[uu][m];
+                mul[m] = 1.f / l;
+            }
+        }
         float ss = 0.f;
 #pragma unroll
         for (int t = 0; t < MAXTV; ++t)
@@ -665,8 +675,10 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
                               int heads, int kv_heads, int maps, int dk, int dv, int block_size, int window,
                               int keep_first, int chunk, float scale, const float* slopes, const float* talk, float lambda,
                               int head_norm, float eps, float out_scale, int shares, float* ws_stats, float* ws_o, int ws_rows,
-                              const float* dist_bias, int dist_reach, const float* gate, int gate_stride, hipStream_t stream) {
+                              const float* dist_bias, int dist_reach, const float* gate, int gate_stride, int sink,
+                              hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && max_new > 0 && heads > 0 && kv_heads > 0, "attend_composed_mfma: sizes must be positive");
+    LLMS_REQUIRE(!(sink && talk), "attend_composed_mfma: no sink where heads are mixed");
     LLMS_REQUIRE(heads % kv_heads == 0 && heads / kv_heads <= 16, "attend_composed_mfma: up to 16 query heads per key/value head");
     LLMS_REQUIRE(maps == 1 || maps == 2, "attend_composed_mfma: one or two score maps");
     LLMS_REQUIRE(!(talk && maps != 1), "attend_composed_mfma: mixing heads' weights goes with one score map");
@@ -685,7 +697,7 @@ int llms_attend_composed_mfma(void* out, int out_stride, const void* q, int q_st
     a.out_stride = out_stride, a.q_stride = q_stride, a.max_blocks = max_blocks, a.seq_begin = seq_begin, a.n_seqs = n_seqs;
     a.heads = heads, a.kv_heads = kv_heads, a.grp = heads / kv_heads, a.dk = dk, a.dv = dv, a.block_size = block_size;
     a.window = window, a.keep_first = keep_first, a.chunk = chunk;
-    a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm;
+    a.scale = scale, a.lambda = lambda, a.eps = eps, a.out_scale = out_scale, a.head_norm = head_norm, a.sink = sink;
     a.tpw = 16 / a.grp;
     a.shares = 1, a.mode = 0, a.ws_stats = ws_stats, a.ws_o = ws_o, a.ws_rows = ws_rows;
     a.bs_magic = (unsigned)((0x100000000ull + block_size - 1) / block_size);

@@ -1163,7 +1163,7 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
                          chunk: int = 0, slopes: torch.Tensor | None = None, talk: torch.Tensor | None = None,
                          lam: float = 0.0, head_norm: bool = False, eps: float = 0.0, out_scale: float = 1.0,
                          table_rows: torch.Tensor | None = None, shares: int = 1, dist_bias: torch.Tensor | None = None,
-                         gate: torch.Tensor | None = None) -> torch.Tensor:
+                         gate: torch.Tensor | None = None, sink: bool = False) -> torch.Tensor:
     """`attend_composed` on the matrix cores (bfloat16) for requests [seq_begin, seq_begin + n_seqs) of a step: request
     b owns rows cu_seqlens[b] .. cu_seqlens[b+1] of q and out, brings at most `max_new` tokens and is context_lens[b]
     long after the step (0: padding, left alone).  Same arguments and arithmetic otherwise; the weights are rounded
@@ -1225,7 +1225,7 @@ def attend_composed_mfma(out: torch.Tensor, q: torch.Tensor, k_pool: torch.Tenso
         c_int(block_size), c_int(window), c_int(keep_first), c_int(chunk), c_float(scale), _ptr(slopes), _ptr(talk),
         c_float(lam), c_int(1 if head_norm else 0), c_float(eps), c_float(out_scale), c_int(shares), _ptr(ws_stats),
         _ptr(ws_o), c_int(q.shape[0]), _ptr(dist_bias), c_int(dist_bias.shape[1] - 1 if dist_bias is not None else 0),
-        _ptr(gate), c_int(gate.stride(0) if gate is not None else 0), _stream(dev)),
+        _ptr(gate), c_int(gate.stride(0) if gate is not None else 0), c_int(1 if sink else 0), _stream(dev)),
         "attend_composed_mfma")
     return out
 

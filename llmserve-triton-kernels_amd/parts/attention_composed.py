@@ -317,7 +317,7 @@ class ComposedAttention(Mixer):
                       keep_first=self.keep_first, chunk=int(self.chunk or 0), slopes=self.slopes, talk=self.talk,
                       lam=self.lam, head_norm=self.head_norm_eps is not None, eps=float(self.head_norm_eps or 0.0),
                       out_scale=self.head_norm_scale, table_rows=batch.state_slots)
-        if self.sink or (gate is not None and (self.talking or gate.data_ptr() % 16 or gate.stride(0) % 4)) or \
+        if (self.sink and self.talking) or (gate is not None and (self.talking or gate.data_ptr() % 16 or gate.stride(0) % 4)) or \
                 not ops.attend_composed_mfma_supported(
                 q.dtype, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, paged.block_size, self.talking):
             ops.attend_composed(out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.token_seq, batch.positions,
@@ -325,7 +325,7 @@ class ComposedAttention(Mixer):
                                 **common)
             return
         args = (out, q, paged.k_pool, paged.v_pool, view.block_tables, batch.cu_seqlens, batch.context_lens)
-        common.update(dist_bias=self.dist_bias, gate=gate)
+        common.update(dist_bias=self.dist_bias, gate=gate, sink=self.sink)
         n_dec = batch.num_decode
         if n_dec:
             ops.attend_composed_mfma(*args, 0, n_dec, 1, shares=self.decode_shares(n_dec, batch.max_decode_context,

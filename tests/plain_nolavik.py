@@ -14,6 +14,15 @@ import torch
 F64 = torch.float64
 
 
+_ROUND = None  # set while `forward(..., rounded=...)` runs
+
+
+def operand(x):
+    """An operand of a sublayer's first or last matrix product: as it is, or rounded where `forward` was asked to show
+    what rounding these operands alone does."""
+    return x if _ROUND is None else _ROUND(x)
+
+
 def rms(x, eps, weight=None):
     y = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
     return y if weight is None else y * weight
@@ -92,7 +101,7 @@ def sink_attention(h, t, p, m, eps):
         e = torch.exp(s)
         w = e / (1.0 + e.sum(-1, keepdim=True))
         out[:, a] = w @ v[:, g]
-    return out.reshape(T, H * dv) @ t[p + "o"].T
+    return operand(out.reshape(T, H * dv)) @ t[p + "o"].T
 
 
 def selective_scan(h, t, p, m):
@@ -111,7 +120,7 @@ def selective_scan(h, t, p, m):
     for i in range(T):
         S = torch.exp(dt[i][:, None] * A) * S + (dt[i] * x[i])[:, None] * B[i][None, :]
         y[i] = S @ C[i] + t[p + "D"] * x[i]
-    return (y * silu(z)) @ t[p + "o"].T
+    return operand(y * silu(z)) @ t[p + "o"].T
 
 
 def parallel_mixer(h, t, p, m, eps):
@@ -141,7 +150,7 @@ def latent_attention(h, t, p, m, eps):
     for a in range(H):
         s = (qn[:, a] @ kn[:, a].T + qr[:, a] @ kr.T) * float(m["scale"])
         out[:, a] = torch.softmax(s.masked_fill(mask, -math.inf), dim=-1) @ v[:, a]
-    return out.reshape(T, H * dv) @ t[p + "o"].T
+    return operand(out.reshape(T, H * dv)) @ t[p + "o"].T
 
 
 def gated_delta(h, t, p, m, eps):
@@ -166,12 +175,12 @@ def gated_delta(h, t, p, m, eps):
             S = S + torch.outer(k[i, g], u)
             out[i, a] = S.T @ q[i, g]
     out = rms(out, eps, t[p + "norm"]) * gate
-    return out.reshape(T, H * dv) @ t[p + "o"].T
+    return operand(out.reshape(T, H * dv)) @ t[p + "o"].T
 
 
 # ------------------------------------------------------------------------------------------------ feed-forward
 def gated_unit(h, t, p):
-    return (silu(h @ t[p + "gate"].T) * (h @ t[p + "up"].T)) @ t[p + "down"].T
+    return operand(silu(h @ t[p + "gate"].T) * (h @ t[p + "up"].T)) @ t[p + "down"].T
 
 
 def route(h, t, p, top):
@@ -195,9 +204,6 @@ def mixture(h, t, p, mlp):
 
 
 # ------------------------------------------------------------------------------------------------ the model
-MIXERS = {"parallel": parallel_mixer, "latent_attention": latent_attention}
-
-
 def mixer(kind, h, t, p, m, eps):
     if kind == "parallel":
         return parallel_mixer(h, t, p, m, eps)
@@ -210,9 +216,9 @@ def mixer(kind, h, t, p, m, eps):
 
 def layer(x, t, i, entry, eps):
     p = f"l{i}."
-    x = x + rms(mixer(entry["type"], rms(x, eps, t[p + "norm1"]), t, p + "mix.", entry["mixer"], eps), eps, t[p + "norm1b"])
+    x = x + rms(mixer(entry["type"], operand(rms(x, eps, t[p + "norm1"])), t, p + "mix.", entry["mixer"], eps), eps, t[p + "norm1b"])
     if entry.get("mlp") is not None:
-        x = x + rms(mixture(rms(x, eps, t[p + "norm2"]), t, p + "mlp.", entry["mlp"]), eps, t[p + "norm2b"])
+        x = x + rms(mixture(operand(rms(x, eps, t[p + "norm2"])), t, p + "mlp.", entry["mlp"]), eps, t[p + "norm2b"])
     return x
 
 
@@ -229,8 +235,18 @@ def layer_runs(config):
     return runs + [(i, None) for i in range(stop, n)]
 
 
-def forward(config, t, tokens, collect=None):
-    """Logits [T, vocab] of one sequence.  `collect`: a list that receives the residual stream after every layer run."""
+def forward(config, t, tokens, collect=None, rounded=None):
+    """Logits [T, vocab] of one sequence.  `collect`: a list that receives the residual stream after every layer run.
+    `rounded`: a function applied to every sublayer's normed input and to the operand of its last matrix product."""
+    global _ROUND
+    _ROUND = rounded
+    try:
+        return _forward(config, t, tokens, collect)
+    finally:
+        _ROUND = None
+
+
+def _forward(config, t, tokens, collect):
     eps = float(config["norm"]["eps"])
     x = t["embed"][torch.as_tensor(tokens, dtype=torch.long)]
     for i, k in layer_runs(config):
