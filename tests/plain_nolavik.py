@@ -18,8 +18,8 @@ _ROUND = None  # set while `forward(..., rounded=...)` runs
 
 
 def operand(x):
-    """An operand of a sublayer's first or last matrix product: as it is, or rounded where `forward` was asked to show
-    what rounding these operands alone does."""
+    """An operand of a matrix product (a sublayer's input, what its last projection reads, queries, keys, values and
+    latents): as it is, or rounded where `forward` was asked to show what rounding these operands alone does."""
     return x if _ROUND is None else _ROUND(x)
 
 
@@ -92,7 +92,7 @@ def sink_attention(h, t, p, m, eps):
     rot = m.get("rot") or {}
     freq = frequencies(rot.get("base", 10000.0), int(rot.get("dims", 0)), rot.get("scaling"))
     pos = torch.arange(T)
-    q, k = rms(rotate_half(q, freq, pos), eps), rms(rotate_half(k, freq, pos), eps)
+    q, k, v = operand(rms(rotate_half(q, freq, pos), eps)), operand(rms(rotate_half(k, freq, pos), eps)), operand(v)
     out = torch.zeros(T, H, dv, dtype=F64)
     for a in range(H):
         g = a // (H // G)
@@ -111,7 +111,7 @@ def selective_scan(h, t, p, m):
     xz = h @ t[p + "in"].T
     x, z = xz[:, :inner], xz[:, inner:]
     x = silu(causal_conv(x, t[p + "conv"], t[p + "conv.b"]))
-    low = x @ t[p + "x"].T
+    low = operand(x) @ t[p + "x"].T
     dt = softplus(low[:, :R] @ t[p + "dt"].T + t[p + "dt.b"][None, :])
     B, C = low[:, R:R + N], low[:, R + N:R + 2 * N]
     A = -torch.exp(t[p + "A_log"])
@@ -137,12 +137,12 @@ def latent_attention(h, t, p, m, eps):
     rot = m.get("rot") or {}
     freq = frequencies(rot.get("base", 10000.0), int(rot.get("dims", dr)), rot.get("scaling"))
     pos = torch.arange(T)
-    cq = rms(h @ t[p + "dq"].T, eps, t[p + "dq.norm"])
+    cq = operand(rms(h @ t[p + "dq"].T, eps, t[p + "dq.norm"]))
     q = (cq @ t[p + "uq"].T).view(T, H, dn + dr)
-    qn, qr = q[..., :dn], rotate_half(q[..., dn:], freq, pos)
+    qn, qr = operand(q[..., :dn]), operand(rotate_half(q[..., dn:], freq, pos))
     kv = h @ t[p + "dkv"].T
-    c = rms(kv[:, :r], eps, t[p + "dkv.norm"])
-    kr = rotate_half(kv[:, r:].reshape(T, 1, dr), freq, pos)[:, 0]
+    c = operand(rms(kv[:, :r], eps, t[p + "dkv.norm"]))
+    kr = operand(rotate_half(kv[:, r:].reshape(T, 1, dr), freq, pos)[:, 0])
     kn = (c @ t[p + "uk"].T).view(T, H, dn)
     v = (c @ t[p + "uv"].T).view(T, H, dv)
     out = torch.zeros(T, H, dv, dtype=F64)
@@ -237,7 +237,7 @@ def layer_runs(config):
 
 def forward(config, t, tokens, collect=None, rounded=None):
     """Logits [T, vocab] of one sequence.  `collect`: a list that receives the residual stream after every layer run.
-    `rounded`: a function applied to every sublayer's normed input and to the operand of its last matrix product."""
+    `rounded`: a function applied to the operands of matrix products (see `operand`)."""
     global _ROUND
     _ROUND = rounded
     try:
