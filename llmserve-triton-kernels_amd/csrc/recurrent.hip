@@ -9,7 +9,10 @@
 //                   token, conv_act writes the ring itself).
 //   selective_scan  per channel c and state n:  S <- exp(dt_c A[c, n]) S + dt_c x_c B_n,  y_c = sum_n S C_n + D_c x_c,
 //                   dt = softplus(dt_raw + bias), and y silu(z) leaves rounded once.  16 lanes share a channel's states.
-//   unit_heads      every head of q and k is divided by sqrt(sum of squares + eps); q is multiplied by a factor.
+//   unit_heads      every head of q and k is divided by sqrt(sum of squares + eps); q is multiplied by a factor; where
+//                   a step brings many tokens it also turns the gates' products into decay and beta, and
+//   scan_prepare    forms the step sizes and silu(z) of the selective scan, so that no logarithm and no exponential
+//                   besides the recurrence's own stands in the chain from token to token.
 //   delta_scan      the gated delta rule per head over a state S [dk, dv]:
 //                   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the token's write)
 //                   with beta = sigmoid(zb) and g = exp(-exp(A_log) softplus(za + dt_bias)).  16 lanes share a column.
@@ -25,6 +28,14 @@
 
 __device__ __forceinline__ float rc_silu(float x) { return x / (1.f + expf(-x)); }
 __device__ __forceinline__ float rc_softplus(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+// exp(x) for the inside of a recurrence, a handful of instructions: 2^(x log2 e) by the hardware's exponential, with the
+// rounding of the product x log2 e put back as a factor (1 + error ln 2); within two units in the last place for x <= 0
+__device__ __forceinline__ float rc_exp(float x) {
+    const float t = x * 1.44269504f;
+    const float err = fmaf(x, 1.92596299e-8f, fmaf(x, 1.44269504f, -t));
+    const float e = __builtin_amdgcn_exp2f(t);
+    return fmaf(e, err * 0.693147181f, e);
+}
 
 // sum over the 16 lanes of a row of the wave, the same value in all of them (no LDS: four lane exchanges inside the row)
 __device__ __forceinline__ float row16_sum(float v) {
@@ -93,7 +104,9 @@ __global__ __launch_bounds__(RC_THREADS) void conv_ring_kernel(
 // grid (requests, channels / 16).  Thread (channel, lane of 16): states lane, lane + 16, ...  R = ceil(states / 16).
 // x [N, x_ld] (after the convolution), z [N, z_ld] columns z_col .., low [N, low_ld]: B at b_col, C at c_col,
 // dt_raw [N, dt_ld]; S [channels, states] at scan_off inside a slot.
-template <typename T, int R>
+// PREP: dt_raw already holds softplus(dt_raw + bias) and z already silu(z) (`scan_prepare`), which keeps the
+// logarithm and the exponentials that do not belong to the recurrence out of its chain.
+template <typename T, int R, bool PREP>
 __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
     T* __restrict__ out, int out_ld, const float* __restrict__ x, int x_ld, const float* __restrict__ z, int z_ld, int z_col,
     const float* __restrict__ low, int low_ld, int b_col, int c_col, const float* __restrict__ dt_raw, int dt_ld,
@@ -116,24 +129,42 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
         a[r] = k < states ? a_neg[(size_t)cc * states + k] : 0.f;
     }
     const float bias = dt_bias[cc], skip = d_skip[cc];
-    for (int t = 0; t < count; ++t) {
-        const size_t row = (size_t)(first_row + t);
-        const float dt = rc_softplus(dt_raw[row * dt_ld + cc] + bias);
-        const float xv = x[row * x_ld + cc];
-        const float dx = dt * xv;
-        float y = 0.f;
+    // tokens in groups of U: what a group reads is asked for before its first token is worked on, so a group costs one
+    // trip to memory and not one per token (the recurrence itself is a chain from token to token)
+    constexpr int U = R <= 2 ? 8 : (R <= 4 ? 4 : 2);
+    for (int t0 = 0; t0 < count; t0 += U) {
+        float dtr[U], xs[U], zs[U], bn[U][R], cn[U][R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int k = lane + 16 * r;
-            const float bn = k < states ? low[row * low_ld + b_col + k] : 0.f;
-            const float cn = k < states ? low[row * low_ld + c_col + k] : 0.f;
-            s[r] = fmaf(expf(dt * a[r]), s[r], dx * bn);
-            y = fmaf(s[r], cn, y);
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u < count ? t0 + u : count - 1;
+            const size_t row = (size_t)(first_row + t);
+            dtr[u] = dt_raw[row * dt_ld + cc];
+            xs[u] = x[row * x_ld + cc];
+            zs[u] = z[row * z_ld + z_col + cc];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int k = lane + 16 * r;
+                bn[u][r] = k < states ? low[row * low_ld + b_col + k] : 0.f;
+                cn[u][r] = k < states ? low[row * low_ld + c_col + k] : 0.f;
+            }
         }
-        y = row16_sum(y);
-        if (lane == 0 && live) {
-            y = fmaf(skip, xv, y);
-            out[row * out_ld + c] = from_f32<T>(y * rc_silu(z[row * z_ld + z_col + c]));
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (t0 + u >= count) break;
+            const size_t row = (size_t)(first_row + t0 + u);
+            const float dt = PREP ? dtr[u] : rc_softplus(dtr[u] + bias);
+            const float dx = dt * xs[u];
+            float y = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                s[r] = fmaf(rc_exp(dt * a[r]), s[r], dx * bn[u][r]);
+                y = fmaf(s[r], cn[u][r], y);
+            }
+            y = row16_sum(y);
+            if (lane == 0 && live) {
+                y = fmaf(skip, xs[u], y);
+                out[row * out_ld + c] = from_f32<T>(y * (PREP ? zs[u] : rc_silu(zs[u])));
+            }
         }
     }
     if (live) {
@@ -145,12 +176,35 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
     }
 }
 
+// grid (tokens, channel blocks): dt_raw <- softplus(dt_raw + bias), z <- silu(z), in place
+__global__ __launch_bounds__(RC_THREADS) void scan_prepare_kernel(float* __restrict__ dt_raw, int dt_ld, const float* __restrict__ dt_bias,
+                                                                 float* __restrict__ z, int z_ld, int z_col, int channels) {
+    const int n = blockIdx.x, c = blockIdx.y * RC_THREADS + threadIdx.x;
+    if (c >= channels) return;
+    dt_raw[(size_t)n * dt_ld + c] = rc_softplus(dt_raw[(size_t)n * dt_ld + c] + dt_bias[c]);
+    float* zp = z + (size_t)n * z_ld + z_col + c;
+    *zp = rc_silu(*zp);
+}
+
 // ------------------------------------------------------------------------------------------- unit heads
 // grid (tokens, heads of q + heads of k): one wave a head, in place on x [N, ld]: q heads at q_col, k heads behind them at k_col
+// A last block per token (with `gates`): gates[n, a_col + h] <- exp(-exp(a_log[h]) softplus(. + dt_bias[h])) and
+// gates[n, b_col + h] <- sigmoid(.), the decay and the step of the delta rule, in place.
 __global__ __launch_bounds__(LLMS_WAVE) void unit_heads_kernel(float* __restrict__ x, int ld, int q_col, int k_col, int q_heads,
-                                                               int k_heads, int dk, float eps, float q_factor) {
+                                                               int k_heads, int dk, float eps, float q_factor,
+                                                               float* __restrict__ gates, int g_ld, int a_col, int b_col,
+                                                               const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                                               int heads) {
     const int n = blockIdx.x, lane = threadIdx.x;
     const int head = blockIdx.y;
+    if (head >= q_heads + k_heads) {
+        float* g = gates + (size_t)n * g_ld;
+        for (int h = lane; h < heads; h += LLMS_WAVE) {
+            g[a_col + h] = expf(-expf(a_log[h]) * rc_softplus(g[a_col + h] + dt_bias[h]));
+            g[b_col + h] = 1.f / (1.f + expf(-g[b_col + h]));
+        }
+        return;
+    }
     const bool is_q = head < q_heads;
     float* v = x + (size_t)n * ld + (is_q ? q_col + head * dk : k_col + (head - q_heads) * dk);
     float ss = 0.f;
@@ -163,7 +217,8 @@ __global__ __launch_bounds__(LLMS_WAVE) void unit_heads_kernel(float* __restrict
 // grid (requests, heads, columns / 16).  Thread (column j, lane of 16): rows lane, lane + 16, ... of column j of S.
 // qkv [N, qkv_ld]: q heads at q_col (kv_heads * dk), k heads at k_col, v heads at v_col (heads * dv), prepared;
 // gates [N, g_ld]: za at a_col + head, zb at b_col + head.  S [heads, dk, dv] at scan_off inside a slot.
-template <int R>
+// PREP: the gates' columns already hold decay and beta (`unit_heads` with gates).
+template <int R, bool PREP>
 __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
     float* __restrict__ o, int o_ld, const float* __restrict__ qkv, int qkv_ld, int q_col, int k_col, int v_col,
     const float* __restrict__ gates, int g_ld, int a_col, int b_col, const float* __restrict__ a_log,
@@ -186,34 +241,47 @@ __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
         s[r] = i < dk ? sh[(size_t)i * dv + jj] : 0.f;
     }
     const float rate = expf(a_log[h]), bias = dt_bias[h];
-    for (int t = 0; t < count; ++t) {
-        const size_t row = (size_t)(first_row + t);
-        const float* qr = qkv + row * qkv_ld + q_col + g * dk;
-        const float* kr = qkv + row * qkv_ld + k_col + g * dk;
-        float kk[R], qq[R];
+    // tokens in groups of U whose inputs are all asked for before the first is worked on (one trip to memory a group)
+    constexpr int U = R <= 4 ? 8 : (R <= 8 ? 4 : 2);
+    for (int t0 = 0; t0 < count; t0 += U) {
+        float kk[U][R], qq[U][R], vs[U], za[U], zb[U];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int i = lane + 16 * r;
-            kk[r] = i < dk ? kr[i] : 0.f;
-            qq[r] = i < dk ? qr[i] : 0.f;
+        for (int u = 0; u < U; ++u) {
+            const int t = t0 + u < count ? t0 + u : count - 1;
+            const size_t row = (size_t)(first_row + t);
+            const float* qr = qkv + row * qkv_ld + q_col + g * dk;
+            const float* kr = qkv + row * qkv_ld + k_col + g * dk;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int i = lane + 16 * r;
+                kk[u][r] = i < dk ? kr[i] : 0.f;
+                qq[u][r] = i < dk ? qr[i] : 0.f;
+            }
+            vs[u] = qkv[row * qkv_ld + v_col + h * dv + jj];
+            za[u] = gates[row * g_ld + a_col + h];
+            zb[u] = gates[row * g_ld + b_col + h];
         }
-        const float v = qkv[row * qkv_ld + v_col + h * dv + jj];
-        const float decay = expf(-rate * rc_softplus(gates[row * g_ld + a_col + h] + bias));
-        const float beta = 1.f / (1.f + expf(-gates[row * g_ld + b_col + h]));
-        // with S' = decay S:  u = beta (v - S'^T k),  o = (S' + k u^T)^T q = S'^T q + (k . q) u
-        float sk = 0.f, sq = 0.f, kq = 0.f;
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            s[r] *= decay;
-            sk = fmaf(s[r], kk[r], sk);
-            sq = fmaf(s[r], qq[r], sq);
-            kq = fmaf(kk[r], qq[r], kq);
+        for (int u = 0; u < U; ++u) {
+            if (t0 + u >= count) break;
+            const size_t row = (size_t)(first_row + t0 + u);
+            const float decay = PREP ? za[u] : expf(-rate * rc_softplus(za[u] + bias));
+            const float beta = PREP ? zb[u] : 1.f / (1.f + expf(-zb[u]));
+            // with S' = decay S:  u = beta (v - S'^T k),  o = (S' + k u^T)^T q = S'^T q + (k . q) u
+            float sk = 0.f, sq = 0.f, kq = 0.f;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                s[r] *= decay;
+                sk = fmaf(s[r], kk[u][r], sk);
+                sq = fmaf(s[r], qq[u][r], sq);
+                kq = fmaf(kk[u][r], qq[u][r], kq);
+            }
+            sk = row16_sum(sk), sq = row16_sum(sq), kq = row16_sum(kq);
+            const float w = beta * (vs[u] - sk);
+#pragma unroll
+            for (int r = 0; r < R; ++r) s[r] = fmaf(kk[u][r], w, s[r]);
+            if (lane == 0 && live) o[row * o_ld + h * dv + j] = fmaf(kq, w, sq);
         }
-        sk = row16_sum(sk), sq = row16_sum(sq), kq = row16_sum(kq);
-        const float u = beta * (v - sk);
-#pragma unroll
-        for (int r = 0; r < R; ++r) s[r] = fmaf(kk[r], u, s[r]);
-        if (lane == 0 && live) o[row * o_ld + h * dv + j] = fmaf(kq, u, sq);
     }
     if (live) {
 #pragma unroll
@@ -279,20 +347,22 @@ int llms_selective_scan(int dtype, void* out, int out_ld, const float* x, int x_
                         const float* low, int low_ld, int b_col, int c_col, const float* dt_raw, int dt_ld,
                         const float* dt_bias, const float* a_neg, const float* d_skip, int channels, int states, float* state,
                         size_t slot_stride, size_t scan_off, const int* state_slots, const int* cu_seqlens,
-                        const int* context_lens, int n_seqs, hipStream_t stream) {
+                        const int* context_lens, int n_seqs, int prepared, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && channels > 0 && states > 0 && states <= 256, "selective_scan: 1 to 256 states per channel");
     LLMS_REQUIRE(dtype == 0 || dtype == 1, "selective_scan: dtype must be 0 (float32) or 1 (bfloat16)");
     dim3 grid(n_seqs, (channels + RC_THREADS / 16 - 1) / (RC_THREADS / 16));
     const int r = (states + 15) / 16;
-#define SCAN_GO(T, R)                                                                                                     \
-    selective_scan_kernel<T, R><<<grid, RC_THREADS, 0, stream>>>((T*)out, out_ld, x, x_ld, z, z_ld, z_col, low, low_ld, b_col, \
-                                                                 c_col, dt_raw, dt_ld, dt_bias, a_neg, d_skip, channels,  \
-                                                                 states, state, slot_stride, scan_off, state_slots,      \
-                                                                 cu_seqlens, context_lens)
+#define SCAN_GO(T, R, P)                                                                                                  \
+    selective_scan_kernel<T, R, P><<<grid, RC_THREADS, 0, stream>>>((T*)out, out_ld, x, x_ld, z, z_ld, z_col, low, low_ld,    \
+                                                                    b_col, c_col, dt_raw, dt_ld, dt_bias, a_neg, d_skip,  \
+                                                                    channels, states, state, slot_stride, scan_off,      \
+                                                                    state_slots, cu_seqlens, context_lens)
 #define SCAN_R(R)                                                                                                         \
     do {                                                                                                                  \
-        if (dtype == 0) SCAN_GO(float, R);                                                                                \
-        else SCAN_GO(bf16, R);                                                                                            \
+        if (dtype == 0 && prepared) SCAN_GO(float, R, true);                                                              \
+        else if (dtype == 0) SCAN_GO(float, R, false);                                                                    \
+        else if (prepared) SCAN_GO(bf16, R, true);                                                                        \
+        else SCAN_GO(bf16, R, false);                                                                                     \
     } while (0)
     if (r <= 1) SCAN_R(1);
     else if (r <= 2) SCAN_R(2);
@@ -305,33 +375,50 @@ int llms_selective_scan(int dtype, void* out, int out_ld, const float* x, int x_
 }
 
 int llms_unit_heads(float* x, int ld, int q_col, int k_col, int q_heads, int k_heads, int dk, float eps, float q_factor,
-                    int n_tokens, hipStream_t stream) {
+                    int n_tokens, float* gates, int g_ld, int a_col, int b_col, const float* a_log, const float* dt_bias,
+                    int heads, hipStream_t stream) {
     LLMS_REQUIRE(n_tokens > 0 && q_heads >= 0 && k_heads >= 0 && q_heads + k_heads > 0 && dk > 0, "unit_heads: sizes must be positive");
-    LLMS_REQUIRE(q_heads + k_heads <= 65535, "unit_heads: up to 65,535 heads in all");
-    dim3 grid(n_tokens, q_heads + k_heads);
-    unit_heads_kernel<<<grid, LLMS_WAVE, 0, stream>>>(x, ld, q_col, k_col, q_heads, k_heads, dk, eps, q_factor);
+    LLMS_REQUIRE(q_heads + k_heads < 65535, "unit_heads: up to 65,534 heads in all");
+    LLMS_REQUIRE(!gates || (a_log && dt_bias && heads > 0), "unit_heads: gates need their rates and biases");
+    dim3 grid(n_tokens, q_heads + k_heads + (gates ? 1 : 0));
+    unit_heads_kernel<<<grid, LLMS_WAVE, 0, stream>>>(x, ld, q_col, k_col, q_heads, k_heads, dk, eps, q_factor, gates, g_ld, a_col,
+                                                      b_col, a_log, dt_bias, heads);
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_scan_prepare(float* dt_raw, int dt_ld, const float* dt_bias, float* z, int z_ld, int z_col, int channels, int n_tokens,
+                      hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && channels > 0, "scan_prepare: sizes must be positive");
+    dim3 grid(n_tokens, (channels + RC_THREADS - 1) / RC_THREADS);
+    scan_prepare_kernel<<<grid, RC_THREADS, 0, stream>>>(dt_raw, dt_ld, dt_bias, z, z_ld, z_col, channels);
     LLMS_LAUNCH_CHECK();
 }
 
 int llms_delta_scan(float* o, int o_ld, const float* qkv, int qkv_ld, int q_col, int k_col, int v_col, const float* gates,
                     int g_ld, int a_col, int b_col, const float* a_log, const float* dt_bias, int heads, int kv_heads, int dk,
                     int dv, float* state, size_t slot_stride, size_t scan_off, const int* state_slots, const int* cu_seqlens,
-                    const int* context_lens, int n_seqs, hipStream_t stream) {
+                    const int* context_lens, int n_seqs, int prepared, hipStream_t stream) {
     LLMS_REQUIRE(n_seqs > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "delta_scan: heads must be a multiple of kv_heads");
     LLMS_REQUIRE(dk > 0 && dk <= 256 && dv > 0, "delta_scan: keys of 1 to 256 numbers");
     LLMS_REQUIRE(heads <= 65535, "delta_scan: up to 65,535 heads");
     dim3 grid(n_seqs, heads, (dv + RC_THREADS / 16 - 1) / (RC_THREADS / 16));
     const int r = (dk + 15) / 16;
+#define DELTA_P(R, P)                                                                                                     \
+    delta_scan_kernel<R, P><<<grid, RC_THREADS, 0, stream>>>(o, o_ld, qkv, qkv_ld, q_col, k_col, v_col, gates, g_ld, a_col,   \
+                                                             b_col, a_log, dt_bias, heads, kv_heads, dk, dv, state,       \
+                                                             slot_stride, scan_off, state_slots, cu_seqlens, context_lens)
 #define DELTA_GO(R)                                                                                                       \
-    delta_scan_kernel<R><<<grid, RC_THREADS, 0, stream>>>(o, o_ld, qkv, qkv_ld, q_col, k_col, v_col, gates, g_ld, a_col, b_col, \
-                                                          a_log, dt_bias, heads, kv_heads, dk, dv, state, slot_stride,    \
-                                                          scan_off, state_slots, cu_seqlens, context_lens)
+    do {                                                                                                                  \
+        if (prepared) DELTA_P(R, true);                                                                                   \
+        else DELTA_P(R, false);                                                                                           \
+    } while (0)
     if (r <= 1) DELTA_GO(1);
     else if (r <= 2) DELTA_GO(2);
     else if (r <= 4) DELTA_GO(4);
     else if (r <= 8) DELTA_GO(8);
     else DELTA_GO(16);
 #undef DELTA_GO
+#undef DELTA_P
     LLMS_LAUNCH_CHECK();
 }
 

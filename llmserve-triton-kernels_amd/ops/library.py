@@ -2055,12 +2055,14 @@ SCAN_MAX_STATES = 256
 
 def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: int, low: torch.Tensor, b_col: int, c_col: int,
                    dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_neg: torch.Tensor, d_skip: torch.Tensor,
-                   state: torch.Tensor, scan_offset: int, batch) -> torch.Tensor:
+                   state: torch.Tensor, scan_offset: int, batch, prepare: bool = False) -> torch.Tensor:
     """Per request, token by token, per channel c and state n:  S[c, n] <- exp(dt_c a_neg[c, n]) S[c, n] + dt_c x_c B_n,
     y_c = sum_n S[c, n] C_n + d_skip[c] x_c, with dt = softplus(dt_raw + dt_bias); out[t, c] = y_c silu(z_c), rounded
     once.  x float32 [N, channels]; z float32 [N, >= z_col + channels]; low float32 [N, >=] with B at b_col and C at
     c_col (`states` numbers each); dt_raw float32 [N, channels]; S float32 [channels, states] at `scan_offset` of the
-    request's slot of `state`, read before the first token and left behind the last."""
+    request's slot of `state`, read before the first token and left behind the last.  `prepare`: a launch of its own
+    first turns dt_raw into the step sizes and z into silu(z), in place (for steps of many tokens: the recurrence is a
+    chain from token to token, and what does not depend on it is better done beside it)."""
     dev = _dev(out, x, z, low, dt_raw, dt_bias, a_neg, d_skip, state)
     n, channels = x.shape
     if a_neg.dim() != 2 or a_neg.shape[0] != channels:
@@ -2082,26 +2084,38 @@ def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: i
     _i32(batch.context_lens, "context_lens")
     if n == 0:
         return out
+    if prepare:
+        _check(load("recurrent").llms_scan_prepare(_ptr(dt_raw), c_int(dt_raw.stride(0)), _ptr(dt_bias), _ptr(z), c_int(z.stride(0)),
+                                                   c_int(z_col), c_int(channels), c_int(n), _stream(dev)), "scan_prepare")
     _check(load("recurrent").llms_selective_scan(
         c_int(_code(out)), _ptr(out), c_int(out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(z), c_int(z.stride(0)),
         c_int(z_col), _ptr(low), c_int(low.stride(0)), c_int(b_col), c_int(c_col), _ptr(dt_raw), c_int(dt_raw.stride(0)),
         _ptr(dt_bias), _ptr(a_neg), _ptr(d_skip), c_int(channels), c_int(states), _ptr(state), c_size_t(slot_stride),
         c_size_t(scan_offset), _ptr(batch.state_slots), _ptr(batch.cu_seqlens), _ptr(batch.context_lens),
-        c_int(batch.num_seqs), _stream(dev)), "selective_scan")
+        c_int(batch.num_seqs), c_int(1 if prepare else 0), _stream(dev)), "selective_scan")
     return out
 
 
 def unit_heads(x: torch.Tensor, *, q_col: int, k_col: int, q_heads: int, k_heads: int, dk: int, eps: float,
-               q_factor: float = 1.0) -> torch.Tensor:
+               q_factor: float = 1.0, gates: dict | None = None) -> torch.Tensor:
     """In place on x (float32 [N, >=]): every head of dk numbers among the q_heads at q_col and the k_heads at k_col is
-    divided by sqrt(its sum of squares + eps); the q heads are also multiplied by q_factor."""
+    divided by sqrt(its sum of squares + eps); the q heads are also multiplied by q_factor.  `gates` (the arguments
+    gates, a_col, b_col, a_log, dt_bias, heads of `delta_scan`): the same launch turns the gates' products into the
+    decay exp(-exp(a_log) softplus(. + dt_bias)) and the step sigmoid(.), in place, for `delta_scan(prepared=True)`."""
     dev = _dev(x)
     n = x.shape[0]
     _f32_matrix(x, "x", n, max(q_col + q_heads * dk, k_col + k_heads * dk))
+    g = gates or {}
+    if gates is not None:
+        _f32_matrix(g["gates"], "gates", n, max(g["a_col"], g["b_col"]) + g["heads"])
+        _f32(g["a_log"], "a_log", g["heads"])
+        _f32(g["dt_bias"], "dt_bias", g["heads"])
     if n:
-        _check(load("recurrent").llms_unit_heads(_ptr(x), c_int(x.stride(0)), c_int(q_col), c_int(k_col), c_int(q_heads),
-                                                 c_int(k_heads), c_int(dk), c_float(eps), c_float(q_factor), c_int(n),
-                                                 _stream(dev)), "unit_heads")
+        _check(load("recurrent").llms_unit_heads(
+            _ptr(x), c_int(x.stride(0)), c_int(q_col), c_int(k_col), c_int(q_heads), c_int(k_heads), c_int(dk), c_float(eps),
+            c_float(q_factor), c_int(n), _ptr(g.get("gates")), c_int(g["gates"].stride(0) if gates else 0), c_int(g.get("a_col", 0)),
+            c_int(g.get("b_col", 0)), _ptr(g.get("a_log")), _ptr(g.get("dt_bias")), c_int(g.get("heads", 0)), _stream(dev)),
+            "unit_heads")
     return x
 
 
@@ -2110,12 +2124,13 @@ DELTA_MAX_KEY = 256
 
 def delta_scan(o: torch.Tensor, qkv: torch.Tensor, *, q_col: int, k_col: int, v_col: int, gates: torch.Tensor, a_col: int,
                b_col: int, a_log: torch.Tensor, dt_bias: torch.Tensor, heads: int, kv_heads: int, dk: int, dv: int,
-               state: torch.Tensor, scan_offset: int, batch) -> torch.Tensor:
+               state: torch.Tensor, scan_offset: int, batch, prepared: bool = False) -> torch.Tensor:
     """The gated delta rule per request, token by token, per head h over S [dk, dv] (q and k from head h / (heads /
     kv_heads)):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with beta = sigmoid(gates[:, b_col + h])
     and g = exp(-exp(a_log[h]) softplus(gates[:, a_col + h] + dt_bias[h])).  qkv float32 [N, >=] holds the prepared q
     (kv_heads * dk at q_col), k (at k_col) and v (heads * dv at v_col); o float32 [N, heads * dv]; S float32 [heads, dk,
-    dv] at `scan_offset` of the request's slot of `state`."""
+    dv] at `scan_offset` of the request's slot of `state`.  `prepared`: the gates' columns already hold decay and beta
+    (`unit_heads` with gates)."""
     dev = _dev(o, qkv, gates, a_log, dt_bias, state)
     n = qkv.shape[0]
     if heads % kv_heads or not 1 <= dk <= DELTA_MAX_KEY:
@@ -2134,7 +2149,8 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, *, q_col: int, k_col: int, v_
         _ptr(o), c_int(o.stride(0)), _ptr(qkv), c_int(qkv.stride(0)), c_int(q_col), c_int(k_col), c_int(v_col), _ptr(gates),
         c_int(gates.stride(0)), c_int(a_col), c_int(b_col), _ptr(a_log), _ptr(dt_bias), c_int(heads), c_int(kv_heads),
         c_int(dk), c_int(dv), _ptr(state), c_size_t(slot_stride), c_size_t(scan_offset), _ptr(batch.state_slots),
-        _ptr(batch.cu_seqlens), _ptr(batch.context_lens), c_int(batch.num_seqs), _stream(dev)), "delta_scan")
+        _ptr(batch.cu_seqlens), _ptr(batch.context_lens), c_int(batch.num_seqs), c_int(1 if prepared else 0), _stream(dev)),
+        "delta_scan")
     return o
 
 

@@ -43,6 +43,7 @@ def _fill_rate(shape, generator, device, options):
 @register_mixer("gated_delta")
 class GatedDelta(Mixer):
     graph_safe = True
+    PREPARE_FROM = 4  # new tokens of the longest portion beyond which the gates are formed by a launch of their own
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -101,12 +102,14 @@ class GatedDelta(Mixer):
         qkv = torch.empty((rows, self.channels), dtype=torch.float32, device=dev)
         ops.conv_act(proj, 0, self.channels, self.taps_w, state=cache.state, ring_offset=self.scan_numbers, batch=batch,
                      out32=qkv)
+        gates = dict(gates=proj, a_col=self.col_a, b_col=self.col_b, a_log=self.a_log, dt_bias=self.dt_bias, heads=self.heads)
+        # (steps of many tokens: decay and beta are formed beside the recurrence, not inside its chain from token to token)
+        many = batch.max_count > self.PREPARE_FROM
         ops.unit_heads(qkv, q_col=0, k_col=self.cq, q_heads=self.kv_heads, k_heads=self.kv_heads, dk=self.dk,
-                       eps=self.unit_eps, q_factor=self.dk ** -0.5)
+                       eps=self.unit_eps, q_factor=self.dk ** -0.5, gates=gates if many else None)
         o = torch.empty((rows, self.cv), dtype=torch.float32, device=dev)
-        ops.delta_scan(o, qkv, q_col=0, k_col=self.cq, v_col=2 * self.cq, gates=proj, a_col=self.col_a, b_col=self.col_b,
-                       a_log=self.a_log, dt_bias=self.dt_bias, heads=self.heads, kv_heads=self.kv_heads, dk=self.dk,
-                       dv=self.dv, state=cache.state, scan_offset=0, batch=batch)
+        ops.delta_scan(o, qkv, q_col=0, k_col=self.cq, v_col=2 * self.cq, kv_heads=self.kv_heads, dk=self.dk, dv=self.dv,
+                       state=cache.state, scan_offset=0, batch=batch, prepared=many, **gates)
         out = torch.empty((rows, self.cv), dtype=x.dtype, device=dev)
         ops.delta_finish(out, o, proj, self.col_g, self.norm_weight, heads=self.heads, dv=self.dv, eps=self.eps)
         return linear(out, self.w_o, out_dtype=self.result_dtype)

@@ -50,6 +50,7 @@ def _fill_skip(shape, generator, device, options):
 @register_mixer("selective_scan")
 class SelectiveScan(Mixer):
     graph_safe = True
+    PREPARE_FROM = 4  # new tokens of the longest portion beyond which step sizes and gate get a launch of their own
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -103,5 +104,5 @@ class SelectiveScan(Mixer):
         dt_raw = ops.gemm_fma(torch.empty((rows, c), dtype=torch.float32, device=dev), low[:, :self.dt_rank], self.w_dt)
         out = torch.empty((rows, c), dtype=x.dtype, device=dev)
         ops.selective_scan(out, x32, xz, c, low, self.dt_rank, self.dt_rank + self.states, dt_raw, self.dt_bias, self.a_neg,
-                           self.skip, cache.state, 0, batch)
+                           self.skip, cache.state, 0, batch, prepare=batch.max_count > self.PREPARE_FROM)
         return linear(out, self.w_o, out_dtype=self.result_dtype)

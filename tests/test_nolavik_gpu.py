@@ -165,8 +165,9 @@ def test_the_selective_scan_whole_and_in_portions(inner, states, rank, taps, dty
             low = dev(x32.double().cpu() @ w["x"].T)
             dt_raw = dev(low.double().cpu()[:, :rank] @ w["dt"].T)
             out = torch.full((n, inner), float("nan"), dtype=dtype, device=DEV)
+            # (portions of several tokens: step sizes and gate formed by a launch of their own, as the part does)
             ops.selective_scan(out, x32, proj, inner, low, rank, rank + states, dt_raw, dev(w["dt.b"]), dev(-torch.exp(w["A_log"])),
-                               dev(w["D"]), state, 0, batch)
+                               dev(w["D"]), state, 0, batch, prepare=n > 2)
             outs.append(out.cpu())
         close(torch.cat(outs), want, dtype, f"portions {portions}", loose=3)
         assert bool(torch.isnan(state[0]).all()) and bool(torch.isnan(state[2]).all())
@@ -226,11 +227,13 @@ def run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, portions):
         proj = dev(proj_all[a: a + n])
         qkv = torch.empty((n, channels), dtype=torch.float32, device=DEV)
         ops.conv_act(proj, 0, channels, taps_w, state=state, ring_offset=scan, batch=batch, out32=qkv)
-        ops.unit_heads(qkv, q_col=0, k_col=cq, q_heads=kv, k_heads=kv, dk=dk, eps=1e-6, q_factor=dk ** -0.5)
+        gates = dict(gates=proj, a_col=channels + cv, b_col=channels + cv + heads, a_log=dev(w["A_log"]), dt_bias=dev(w["dt_bias"]),
+                     heads=heads)
+        many = n > 2  # (decay and beta formed beside the recurrence, as the part does for portions of several tokens)
+        ops.unit_heads(qkv, q_col=0, k_col=cq, q_heads=kv, k_heads=kv, dk=dk, eps=1e-6, q_factor=dk ** -0.5, gates=gates if many else None)
         o = torch.full((n, cv), float("nan"), dtype=torch.float32, device=DEV)
-        ops.delta_scan(o, qkv, q_col=0, k_col=cq, v_col=2 * cq, gates=proj, a_col=channels + cv, b_col=channels + cv + heads,
-                       a_log=dev(w["A_log"]), dt_bias=dev(w["dt_bias"]), heads=heads, kv_heads=kv, dk=dk, dv=dv, state=state,
-                       scan_offset=0, batch=batch)
+        ops.delta_scan(o, qkv, q_col=0, k_col=cq, v_col=2 * cq, kv_heads=kv, dk=dk, dv=dv, state=state, scan_offset=0, batch=batch,
+                       prepared=many, **gates)
         out = torch.full((n, cv), float("nan"), dtype=dtype, device=DEV)
         ops.delta_finish(out, o, proj, channels, dev(w["norm"]), heads=heads, dv=dv, eps=eps)
         outs.append(out.cpu())
@@ -581,8 +584,12 @@ def test_the_stream_after_every_layer_run(models, name):
             model._shift(x, delta, model._shift_rows[pos])
         x, delta = model.blocks[index].forward(x, delta, batch, runner.storage.layer_cache(pos, sources[pos]))
         joined = pn.rms(delta.y.double().cpu(), delta.eps, delta.weight.double().cpu())
-        # (a norm behind every sublayer carries a small result's rounding into the stream at full size)
-        close(x[:, 0].double().cpu() + joined, want[pos], torch.float32, f"after layer run {pos}", loose=4)
+        # per token, against the root mean square of the stream: the median token within rounding, and no token far off (a
+        # norm behind every sublayer carries the rounding of a small result into the stream at full size)
+        got = x[:, 0].double().cpu() + joined
+        err = (got - want[pos]).pow(2).mean(-1).sqrt() / want[pos].pow(2).mean().sqrt()
+        assert torch.isfinite(got).all() and float(err.median()) <= 2e-5 and float(err.max()) <= 5e-4, \
+            f"after layer run {pos}: median {float(err.median()):.2e}, worst {float(err.max()):.2e}"
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
