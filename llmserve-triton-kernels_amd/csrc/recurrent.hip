@@ -129,42 +129,71 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
         a[r] = k < states ? a_neg[(size_t)cc * states + k] : 0.f;
     }
     const float bias = dt_bias[cc], skip = d_skip[cc];
-    // tokens in groups of U: what a group reads is asked for before its first token is worked on, so a group costs one
-    // trip to memory and not one per token (the recurrence itself is a chain from token to token)
+    // tokens in groups of U, two groups in registers: the next group is asked for before the present one is worked on, so
+    // the chain from token to token never waits for memory
     constexpr int U = R <= 2 ? 8 : (R <= 4 ? 4 : 2);
-    for (int t0 = 0; t0 < count; t0 += U) {
+    struct Group {
         float dtr[U], xs[U], zs[U], bn[U][R], cn[U][R];
+    };
+    auto fetch = [&](Group& g, int t0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int t = t0 + u < count ? t0 + u : count - 1;
+            int t = t0 + u < count ? t0 + u : count - 1;
             const size_t row = (size_t)(first_row + t);
-            dtr[u] = dt_raw[row * dt_ld + cc];
-            xs[u] = x[row * x_ld + cc];
-            zs[u] = z[row * z_ld + z_col + cc];
+            g.dtr[u] = dt_raw[row * dt_ld + cc];
+            g.xs[u] = x[row * x_ld + cc];
+            g.zs[u] = z[row * z_ld + z_col + cc];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int k = lane + 16 * r;
-                bn[u][r] = k < states ? low[row * low_ld + b_col + k] : 0.f;
-                cn[u][r] = k < states ? low[row * low_ld + c_col + k] : 0.f;
+                g.bn[u][r] = k < states ? low[row * low_ld + b_col + k] : 0.f;
+                g.cn[u][r] = k < states ? low[row * low_ld + c_col + k] : 0.f;
             }
         }
+    };
+    // (results wait in registers and leave four groups at a time: loads and stores share one counter of what is in
+    // flight, and a wait for loads that has stores before it waits for everything, the next group's loads too)
+    float held[4 * U];
+    auto work = [&](const Group& g, int t0, int slot) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (t0 + u >= count) break;
-            const size_t row = (size_t)(first_row + t0 + u);
-            const float dt = PREP ? dtr[u] : rc_softplus(dtr[u] + bias);
-            const float dx = dt * xs[u];
+            const float dt = PREP ? g.dtr[u] : rc_softplus(g.dtr[u] + bias);
+            const float dx = dt * g.xs[u];
             float y = 0.f;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
-                s[r] = fmaf(rc_exp(dt * a[r]), s[r], dx * bn[u][r]);
-                y = fmaf(s[r], cn[u][r], y);
+                s[r] = fmaf(rc_exp(dt * a[r]), s[r], dx * g.bn[u][r]);
+                y = fmaf(s[r], g.cn[u][r], y);
             }
-            y = row16_sum(y);
-            if (lane == 0 && live) {
-                y = fmaf(skip, xs[u], y);
-                out[row * out_ld + c] = from_f32<T>(y * (PREP ? zs[u] : rc_silu(zs[u])));
-            }
+            y = fmaf(skip, g.xs[u], row16_sum(y));
+            held[slot * U + u] = y * (PREP ? g.zs[u] : rc_silu(g.zs[u]));
+        }
+    };
+    auto leave = [&](int t0, int n) {
+        if (lane == 0 && live) {
+#pragma unroll
+            for (int i = 0; i < 4 * U; ++i)
+                if (i < n && t0 + i < count) out[(size_t)(first_row + t0 + i) * out_ld + c] = from_f32<T>(held[i]);
+        }
+    };
+    Group ga;
+    fetch(ga, 0);
+    if (count <= U) {  // (decoding, short portions: one group and no more)
+        work(ga, 0, 0);
+        leave(0, U);
+    } else {
+        Group gb;
+        for (int t0 = 0; t0 < count; t0 += 4 * U) {
+            fetch(gb, t0 + U);  // (a group beyond the last reads the last token again: no branch stands around a load)
+            work(ga, t0, 0);
+            fetch(ga, t0 + 2 * U);
+            work(gb, t0 + U, 1);
+            fetch(gb, t0 + 3 * U);
+            work(ga, t0 + 2 * U, 2);
+            fetch(ga, t0 + 4 * U);
+            work(gb, t0 + 3 * U, 3);
+            leave(t0, 4 * U);
         }
     }
     if (live) {
@@ -217,8 +246,9 @@ __global__ __launch_bounds__(LLMS_WAVE) void unit_heads_kernel(float* __restrict
 // grid (requests, heads, columns / 16).  Thread (column j, lane of 16): rows lane, lane + 16, ... of column j of S.
 // qkv [N, qkv_ld]: q heads at q_col (kv_heads * dk), k heads at k_col, v heads at v_col (heads * dv), prepared;
 // gates [N, g_ld]: za at a_col + head, zb at b_col + head.  S [heads, dk, dv] at scan_off inside a slot.
-// PREP: the gates' columns already hold decay and beta (`unit_heads` with gates).
-template <int R, bool PREP>
+// PREP: the gates' columns already hold decay and beta (`unit_heads` with gates).  VEC: a lane's R rows (R lane .. R lane
+// + R - 1, neighbours, so that k and q arrive in 16-byte pieces) are read four at a time.
+template <int R, bool PREP, bool VEC>
 __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
     float* __restrict__ o, int o_ld, const float* __restrict__ qkv, int qkv_ld, int q_col, int k_col, int v_col,
     const float* __restrict__ gates, int g_ld, int a_col, int b_col, const float* __restrict__ a_log,
@@ -233,62 +263,102 @@ __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
     const bool live = j < dv;
     const int jj = live ? j : dv - 1;
     const int g = h / (heads / kv_heads);
+    const int i0 = R * lane;  // this lane's first row
     float* sh = state + (size_t)state_slots[b] * slot_stride + scan_off + (size_t)h * dk * dv;
     float s[R];
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int i = lane + 16 * r;
-        s[r] = i < dk ? sh[(size_t)i * dv + jj] : 0.f;
-    }
+    for (int r = 0; r < R; ++r) s[r] = i0 + r < dk ? sh[(size_t)(i0 + r) * dv + jj] : 0.f;
     const float rate = expf(a_log[h]), bias = dt_bias[h];
-    // tokens in groups of U whose inputs are all asked for before the first is worked on (one trip to memory a group)
+    // tokens in groups of U, two groups in registers: the next group is asked for before the present one is worked on
     constexpr int U = R <= 4 ? 8 : (R <= 8 ? 4 : 2);
-    for (int t0 = 0; t0 < count; t0 += U) {
+    struct Group {
         float kk[U][R], qq[U][R], vs[U], za[U], zb[U];
+    };
+    const float* q_at = qkv + (size_t)first_row * qkv_ld + q_col + g * dk + i0;
+    const float* k_at = qkv + (size_t)first_row * qkv_ld + k_col + g * dk + i0;
+    const float* v_at = qkv + (size_t)first_row * qkv_ld + v_col + h * dv + jj;
+    const float* a_at = gates + (size_t)first_row * g_ld + a_col + h;
+    const float* b_at = gates + (size_t)first_row * g_ld + b_col + h;
+    auto fetch = [&](Group& gr, int t0) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int t = t0 + u < count ? t0 + u : count - 1;
-            const size_t row = (size_t)(first_row + t);
-            const float* qr = qkv + row * qkv_ld + q_col + g * dk;
-            const float* kr = qkv + row * qkv_ld + k_col + g * dk;
+            const float* qr = q_at + (size_t)t * qkv_ld;
+            const float* kr = k_at + (size_t)t * qkv_ld;
+            if constexpr (VEC) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int i = lane + 16 * r;
-                kk[u][r] = i < dk ? kr[i] : 0.f;
-                qq[u][r] = i < dk ? qr[i] : 0.f;
+                for (int r = 0; r < R; r += 4) {
+                    const bool in = i0 + r < dk;  // (dk is a multiple of 4 here: four rows are inside or outside together)
+                    const float4 kv = in ? *reinterpret_cast<const float4*>(kr + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    const float4 qv = in ? *reinterpret_cast<const float4*>(qr + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    gr.kk[u][r] = kv.x, gr.kk[u][r + 1] = kv.y, gr.kk[u][r + 2] = kv.z, gr.kk[u][r + 3] = kv.w;
+                    gr.qq[u][r] = qv.x, gr.qq[u][r + 1] = qv.y, gr.qq[u][r + 2] = qv.z, gr.qq[u][r + 3] = qv.w;
+                }
+            } else {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    gr.kk[u][r] = i0 + r < dk ? kr[r] : 0.f;
+                    gr.qq[u][r] = i0 + r < dk ? qr[r] : 0.f;
+                }
             }
-            vs[u] = qkv[row * qkv_ld + v_col + h * dv + jj];
-            za[u] = gates[row * g_ld + a_col + h];
-            zb[u] = gates[row * g_ld + b_col + h];
+            gr.vs[u] = v_at[(size_t)t * qkv_ld];
+            gr.za[u] = a_at[(size_t)t * g_ld];
+            gr.zb[u] = b_at[(size_t)t * g_ld];
         }
+    };
+    float held[4 * U];  // (results wait in registers and leave up to four groups at a time)
+    auto work = [&](const Group& gr, int t0, int slot) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (t0 + u >= count) break;
-            const size_t row = (size_t)(first_row + t0 + u);
-            const float decay = PREP ? za[u] : expf(-rate * rc_softplus(za[u] + bias));
-            const float beta = PREP ? zb[u] : 1.f / (1.f + expf(-zb[u]));
+            const float decay = PREP ? gr.za[u] : expf(-rate * rc_softplus(gr.za[u] + bias));
+            const float beta = PREP ? gr.zb[u] : 1.f / (1.f + expf(-gr.zb[u]));
             // with S' = decay S:  u = beta (v - S'^T k),  o = (S' + k u^T)^T q = S'^T q + (k . q) u
             float sk = 0.f, sq = 0.f, kq = 0.f;
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 s[r] *= decay;
-                sk = fmaf(s[r], kk[u][r], sk);
-                sq = fmaf(s[r], qq[u][r], sq);
-                kq = fmaf(kk[u][r], qq[u][r], kq);
+                sk = fmaf(s[r], gr.kk[u][r], sk);
+                sq = fmaf(s[r], gr.qq[u][r], sq);
+                kq = fmaf(gr.kk[u][r], gr.qq[u][r], kq);
             }
             sk = row16_sum(sk), sq = row16_sum(sq), kq = row16_sum(kq);
-            const float w = beta * (vs[u] - sk);
+            const float w = beta * (gr.vs[u] - sk);
 #pragma unroll
-            for (int r = 0; r < R; ++r) s[r] = fmaf(kk[u][r], w, s[r]);
-            if (lane == 0 && live) o[row * o_ld + h * dv + j] = fmaf(kq, w, sq);
+            for (int r = 0; r < R; ++r) s[r] = fmaf(gr.kk[u][r], w, s[r]);
+            held[slot * U + u] = fmaf(kq, w, sq);
+        }
+    };
+    auto leave = [&](int t0, int n) {
+        if (lane == 0 && live) {
+#pragma unroll
+            for (int i = 0; i < 4 * U; ++i)
+                if (i < n && t0 + i < count) o[(size_t)(first_row + t0 + i) * o_ld + h * dv + j] = held[i];
+        }
+    };
+    Group ga;
+    fetch(ga, 0);
+    if (count <= U) {  // (decoding, short portions: one group and no more)
+        work(ga, 0, 0);
+        leave(0, U);
+    } else {
+        Group gb;
+        for (int t0 = 0; t0 < count; t0 += 4 * U) {
+            fetch(gb, t0 + U);  // (a group beyond the last reads the last token again: no branch stands around a load)
+            work(ga, t0, 0);
+            fetch(ga, t0 + 2 * U);
+            work(gb, t0 + U, 1);
+            fetch(gb, t0 + 3 * U);
+            work(ga, t0 + 2 * U, 2);
+            fetch(ga, t0 + 4 * U);
+            work(gb, t0 + 3 * U, 3);
+            leave(t0, 4 * U);
         }
     }
     if (live) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int i = lane + 16 * r;
-            if (i < dk) sh[(size_t)i * dv + j] = s[r];
-        }
+        for (int r = 0; r < R; ++r)
+            if (i0 + r < dk) sh[(size_t)(i0 + r) * dv + j] = s[r];
     }
 }
 
@@ -403,14 +473,18 @@ int llms_delta_scan(float* o, int o_ld, const float* qkv, int qkv_ld, int q_col,
     LLMS_REQUIRE(heads <= 65535, "delta_scan: up to 65,535 heads");
     dim3 grid(n_seqs, heads, (dv + RC_THREADS / 16 - 1) / (RC_THREADS / 16));
     const int r = (dk + 15) / 16;
-#define DELTA_P(R, P)                                                                                                     \
-    delta_scan_kernel<R, P><<<grid, RC_THREADS, 0, stream>>>(o, o_ld, qkv, qkv_ld, q_col, k_col, v_col, gates, g_ld, a_col,   \
-                                                             b_col, a_log, dt_bias, heads, kv_heads, dk, dv, state,       \
-                                                             slot_stride, scan_off, state_slots, cu_seqlens, context_lens)
+    // rows in 16-byte pieces where a lane's rows come in fours and every piece is aligned
+    const bool vec = r % 4 == 0 && dk % 4 == 0 && qkv_ld % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0 && ((uintptr_t)qkv % 16) == 0;
+#define DELTA_P(R, P, V)                                                                                                  \
+    delta_scan_kernel<R, P, V><<<grid, RC_THREADS, 0, stream>>>(o, o_ld, qkv, qkv_ld, q_col, k_col, v_col, gates, g_ld, a_col, \
+                                                                b_col, a_log, dt_bias, heads, kv_heads, dk, dv, state,    \
+                                                                slot_stride, scan_off, state_slots, cu_seqlens, context_lens)
 #define DELTA_GO(R)                                                                                                       \
     do {                                                                                                                  \
-        if (prepared) DELTA_P(R, true);                                                                                   \
-        else DELTA_P(R, false);                                                                                           \
+        if (prepared && vec && R % 4 == 0) DELTA_P(R, true, (R % 4 == 0));                                                \
+        else if (prepared) DELTA_P(R, true, false);                                                                       \
+        else if (vec && R % 4 == 0) DELTA_P(R, false, (R % 4 == 0));                                                      \
+        else DELTA_P(R, false, false);                                                                                    \
     } while (0)
     if (r <= 1) DELTA_GO(1);
     else if (r <= 2) DELTA_GO(2);
