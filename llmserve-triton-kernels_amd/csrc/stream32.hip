@@ -430,7 +430,9 @@ __global__ void weighted_sum_kernel(float* out, const float* a, const float* b, 
     if (i < total) out[i] = fmaf(sa, a[i], sb * b[i]);
 }
 
-// grid: rows.  Dynamic LDS: hidden floats (the summed row).  `y` null: nothing joins; `out` null: the sum alone.
+// grid: rows.  Dynamic LDS: hidden floats (the summed row; rows of up to 4,096 numbers in 16-byte pieces stay in
+// registers instead).  `y` null: nothing joins; `out` null: the sum alone.
+#define NAN_VEC 4
 template <typename T>
 __global__ __launch_bounds__(S32_THREADS) void normed_add_norm_kernel(T* __restrict__ out, float* __restrict__ x,
                                                                       const float* __restrict__ y, const float* __restrict__ wb,
@@ -442,7 +444,55 @@ __global__ __launch_bounds__(S32_THREADS) void normed_add_norm_kernel(T* __restr
     const size_t src = rows ? (size_t)rows[r] : (size_t)r;
     float* xr = x + src * hidden;
     const float* yr = y ? y + src * hidden : nullptr;
-    const bool vec = hidden % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)wb % 16) == 0;
+    const bool vec = hidden % 4 == 0 && ((uintptr_t)x % 16) == 0 && ((uintptr_t)y % 16) == 0 && ((uintptr_t)wb % 16) == 0 &&
+                     ((uintptr_t)w % 16) == 0 && ((uintptr_t)out % 16) == 0;
+    if (vec && hidden <= 4 * NAN_VEC * S32_THREADS) {
+        // the row, what joins it and that norm's weight in registers, all asked for at once: one trip to memory
+        float4 xv[NAN_VEC], yv[NAN_VEC], bv[NAN_VEC];
+#pragma unroll
+        for (int i = 0; i < NAN_VEC; ++i) {
+            const int c = 4 * (threadIdx.x + i * S32_THREADS);
+            const bool in = c < hidden;
+            xv[i] = in ? *reinterpret_cast<const float4*>(xr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            yv[i] = (in && yr) ? *reinterpret_cast<const float4*>(yr + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+            bv[i] = (in && yr) ? *reinterpret_cast<const float4*>(wb + c) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        if (yr) {
+            float sy = 0.f;
+#pragma unroll
+            for (int i = 0; i < NAN_VEC; ++i)
+                sy = fmaf(yv[i].x, yv[i].x, sy), sy = fmaf(yv[i].y, yv[i].y, sy), sy = fmaf(yv[i].z, yv[i].z, sy), sy = fmaf(yv[i].w, yv[i].w, sy);
+            const float inv_y = 1.f / sqrtf(block_sum(sy, red) / (float)hidden + eps_y);
+#pragma unroll
+            for (int i = 0; i < NAN_VEC; ++i) {
+                xv[i].x += yv[i].x * inv_y * bv[i].x, xv[i].y += yv[i].y * inv_y * bv[i].y;
+                xv[i].z += yv[i].z * inv_y * bv[i].z, xv[i].w += yv[i].w * inv_y * bv[i].w;
+                const int c = 4 * (threadIdx.x + i * S32_THREADS);
+                if (store && c < hidden) *reinterpret_cast<float4*>(xr + c) = xv[i];
+            }
+        }
+        if (!out) return;
+        float sx = 0.f;
+#pragma unroll
+        for (int i = 0; i < NAN_VEC; ++i)
+            sx = fmaf(xv[i].x, xv[i].x, sx), sx = fmaf(xv[i].y, xv[i].y, sx), sx = fmaf(xv[i].z, xv[i].z, sx), sx = fmaf(xv[i].w, xv[i].w, sx);
+        const float inv = 1.f / sqrtf(block_sum(sx, red) / (float)hidden + eps);
+        T* orow = out + (size_t)r * hidden;
+#pragma unroll
+        for (int i = 0; i < NAN_VEC; ++i) {
+            const int c = 4 * (threadIdx.x + i * S32_THREADS);
+            if (c >= hidden) continue;
+            const float4 wv = *reinterpret_cast<const float4*>(w + c);
+            const float a = xv[i].x * inv * wv.x, b = xv[i].y * inv * wv.y, cc = xv[i].z * inv * wv.z, d = xv[i].w * inv * wv.w;
+            if constexpr (sizeof(T) == 2) {
+                uint2 packed = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
+                *reinterpret_cast<uint2*>(orow + c) = packed;
+            } else {
+                *reinterpret_cast<float4*>(orow + c) = make_float4(a, b, cc, d);
+            }
+        }
+        return;
+    }
     float inv_y = 0.f;
     if (yr) {
         float ss = 0.f;
