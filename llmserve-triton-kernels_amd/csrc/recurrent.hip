@@ -245,7 +245,8 @@ __global__ __launch_bounds__(LLMS_WAVE) void unit_heads_kernel(float* __restrict
 // ------------------------------------------------------------------------------------------- delta rule
 // grid (requests, heads, columns / 16).  Thread (column j, lane of 16): rows lane, lane + 16, ... of column j of S.
 // qkv [N, qkv_ld]: q heads at q_col (kv_heads * dk), k heads at k_col, v heads at v_col (heads * dv), prepared;
-// gates [N, g_ld]: za at a_col + head, zb at b_col + head.  S [heads, dk, dv] at scan_off inside a slot.
+// gates [N, g_ld]: za at a_col + head, zb at b_col + head.  S at scan_off inside a slot, [heads][dv][dk] (a head's state
+// column by column).
 // PREP: the gates' columns already hold decay and beta (`unit_heads` with gates).  VEC: a lane's R rows (R lane .. R lane
 // + R - 1, neighbours, so that k and q arrive in 16-byte pieces) are read four at a time.
 template <int R, bool PREP, bool VEC>
@@ -264,10 +265,21 @@ __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
     const int jj = live ? j : dv - 1;
     const int g = h / (heads / kv_heads);
     const int i0 = R * lane;  // this lane's first row
+    // a head's state lies column by column ([dv][dk]): a lane's rows are neighbours in memory, a wave reads whole lines
     float* sh = state + (size_t)state_slots[b] * slot_stride + scan_off + (size_t)h * dk * dv;
+    float* scol = sh + (size_t)jj * dk + i0;
+    const bool svec = VEC && ((uintptr_t)sh % 16) == 0;  // (dk is a multiple of 4 with VEC)
     float s[R];
+    if (svec) {
 #pragma unroll
-    for (int r = 0; r < R; ++r) s[r] = i0 + r < dk ? sh[(size_t)(i0 + r) * dv + jj] : 0.f;
+        for (int r = 0; r < R; r += 4) {
+            const float4 v = i0 + r < dk ? *reinterpret_cast<const float4*>(scol + r) : make_float4(0.f, 0.f, 0.f, 0.f);
+            s[r] = v.x, s[r + 1 < R ? r + 1 : r] = v.y, s[r + 2 < R ? r + 2 : r] = v.z, s[r + 3 < R ? r + 3 : r] = v.w;
+        }
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) s[r] = i0 + r < dk ? scol[r] : 0.f;
+    }
     const float rate = expf(a_log[h]), bias = dt_bias[h];
     // tokens in groups of U, two groups in registers: the next group is asked for before the present one is worked on
     constexpr int U = R <= 4 ? 8 : (R <= 8 ? 4 : 2);
@@ -355,10 +367,15 @@ __global__ __launch_bounds__(RC_THREADS) void delta_scan_kernel(
             leave(t0, 4 * U);
         }
     }
-    if (live) {
+    if (live && svec) {
+#pragma unroll
+        for (int r = 0; r < R; r += 4)
+            if (i0 + r < dk)
+                *reinterpret_cast<float4*>(scol + r) = make_float4(s[r], s[r + 1 < R ? r + 1 : r], s[r + 2 < R ? r + 2 : r], s[r + 3 < R ? r + 3 : r]);
+    } else if (live) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
-            if (i0 + r < dk) sh[(size_t)(i0 + r) * dv + j] = s[r];
+            if (i0 + r < dk) scol[r] = s[r];
     }
 }
 

@@ -2128,8 +2128,8 @@ def delta_scan(o: torch.Tensor, qkv: torch.Tensor, *, q_col: int, k_col: int, v_
     """The gated delta rule per request, token by token, per head h over S [dk, dv] (q and k from head h / (heads /
     kv_heads)):  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with beta = sigmoid(gates[:, b_col + h])
     and g = exp(-exp(a_log[h]) softplus(gates[:, a_col + h] + dt_bias[h])).  qkv float32 [N, >=] holds the prepared q
-    (kv_heads * dk at q_col), k (at k_col) and v (heads * dv at v_col); o float32 [N, heads * dv]; S float32 [heads, dk,
-    dv] at `scan_offset` of the request's slot of `state`.  `prepared`: the gates' columns already hold decay and beta
+    (kv_heads * dk at q_col), k (at k_col) and v (heads * dv at v_col); o float32 [N, heads * dv]; S float32 [heads, dv,
+    dk] (a head's state column by column) at `scan_offset` of the request's slot of `state`.  `prepared`: the gates' columns already hold decay and beta
     (`unit_heads` with gates)."""
     dev = _dev(o, qkv, gates, a_log, dt_bias, state)
     n = qkv.shape[0]

@@ -267,8 +267,8 @@ def test_the_read_out_sees_the_tokens_own_write():
                    dt_bias=dev(torch.zeros(1, dtype=F64)), heads=1, kv_heads=1, dk=dk, dv=dv, state=state, scan_offset=0,
                    batch=step_of([1], [1], [0]))
     close(o[0], 0.5 * torch.arange(1, dv + 1, dtype=F64), torch.float32, "the first token's result")
-    # and the state holds k u^T
-    close(state.view(dk, dv), torch.outer(qkv[0, dk: 2 * dk], 0.5 * qkv[0, 2 * dk:]), torch.float32, "the state")
+    # and the state holds k u^T (kept column by column)
+    close(state.view(dv, dk).t(), torch.outer(qkv[0, dk: 2 * dk], 0.5 * qkv[0, 2 * dk:]), torch.float32, "the state")
 
 
 # ------------------------------------------------------------------------------ attention with a sink
