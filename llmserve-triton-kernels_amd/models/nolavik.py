@@ -49,8 +49,8 @@ def _check_rot(where: str, rot: dict, within: int) -> None:
     scaling = rot.get("scaling")
     if scaling:
         missing = [k for k in ("factor", "low", "high", "original") if k not in scaling]
-        if missing or float(scaling["high"]) == float(scaling["low"]):
-            raise ConfigError(f"{where}.rot.scaling needs factor, low, high (different from low) and original")
+        if missing or float(scaling["high"]) == float(scaling["low"]) or float(scaling["factor"]) <= 0:
+            raise ConfigError(f"{where}.rot.scaling needs a positive factor, low, high (different from low) and original")
 
 
 @dataclass(frozen=True)
@@ -227,6 +227,8 @@ def nolavik_spec(cfg: NolavikConfig) -> ModelSpec:
     shifts = tuple((pos, t) for pos, (_layer, t) in enumerate(runs) if t is not None)
     if shifts:
         weights["shifts"] = "loop.step"
+    else:  # (a checkpoint of a model without a loop may hold the tensor all the same)
+        unused.append("loop.step")
     return ModelSpec(
         hidden_size=w, vocab_size=cfg.vocab, max_positions=cfg.max_positions,
         embedding=PartSpec("embedding", {"vocab": cfg.vocab, "hidden": w, "stream": "float32", "tensor": ""}),

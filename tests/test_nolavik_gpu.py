@@ -343,7 +343,7 @@ def test_turned_and_normed_queries_and_keys_and_the_sink(dtype, heads, kv, dk, d
 
 
 MATRIX_CORE_CASES = [  # heads, kv_heads, dk, dv, turned dimensions, stretched, block size, tokens
-    (4, 2, 128, 64, 64, SCALING, 16, 300),
+    (6, 2, 128, 96, 32, SCALING, 16, 300),
     (8, 1, 64, 64, 32, None, 16, 420),
     (6, 3, 80, 48, 16, SCALING, 8, 150),
     (3, 3, 32, 16, 32, None, 4, 70),
@@ -650,6 +650,28 @@ def test_long_decoding_and_the_prompt_of_the_same_tokens_agree(models):
         logits_close(got["long"], ref, torch.float32, "long decoding")
         whole = run_trace(runner, traces.whole({"again": ids}))
         logits_close(whole["again"], ref, torch.float32, "the whole prompt on the slot and pages that came back")
+
+
+@pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
+def test_a_long_request_at_matrix_core_sizes(models, dtype_name):
+    """650 tokens through every kind of layer at sizes the matrix-core kernels take: the prompt in one step and its last
+    tokens one by one (keys shared out to several workgroups, several tiles a wave), then in portions on the pages
+    and the slot that came back."""
+    from llmserve.config import EngineConfig
+    from llmserve.engine.runner import ModelRunner
+
+    folder, config, w, bs = models["small_d"]
+    dtype = getattr(torch, dtype_name)
+    ids = traces.random_ids(config["vocab"], 650, 78)
+    ref = pn.forward(config, w, ids)
+    noise = pn.forward(config, w, ids, rounded=bf16) if dtype == torch.bfloat16 else None
+    runner = ModelRunner.from_folder(folder, EngineConfig(dtype=dtype_name, block_size=bs, num_blocks=-(-650 // bs) + 1,
+                                                          max_num_seqs=2))
+    poison(runner)
+    got = run_trace(runner, traces.prefill_then_decode({"long": ids}, tail=48))
+    logits_close(got["long"], ref, dtype, f"a long prompt, then token by token, {dtype_name}", noise)
+    again = run_trace(runner, traces.portions({"again": ids}, sizes=[200, 7, 2, 130, 64, 1, 33]))
+    logits_close(again["again"], ref, dtype, f"the same in portions, {dtype_name}", noise)
 
 
 @pytest.mark.parametrize("dtype_name", ["float32", "bfloat16"])
