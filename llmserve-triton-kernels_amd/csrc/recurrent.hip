@@ -9,6 +9,7 @@
 //                   token, conv_act writes the ring itself).
 //   selective_scan  per channel c and state n:  S <- exp(dt_c A[c, n]) S + dt_c x_c B_n,  y_c = sum_n S C_n + D_c x_c,
 //                   dt = softplus(dt_raw + bias), and y silu(z) leaves rounded once.  16 lanes share a channel's states.
+//   conv_heads      conv_act and unit_heads in one launch, a wave a head: what the delta rule's layer runs.
 //   unit_heads      every head of q and k is divided by sqrt(sum of squares + eps); q is multiplied by a factor; where
 //                   a step brings many tokens it also turns the gates' products into decay and beta, and
 //   scan_prepare    forms the step sizes and silu(z) of the selective scan, so that no logarithm and no exponential
@@ -48,37 +49,94 @@ __device__ __forceinline__ float row16_sum(float v) {
 
 // ------------------------------------------------------------------------------------------- convolution
 // grid (tokens, channel blocks).  u [N, u_ld] columns u_col ..; ring [taps - 1, channels] at ring_off inside a slot.
-template <typename T>
-__global__ __launch_bounds__(RC_THREADS) void conv_act_kernel(
-    float* __restrict__ y32, int y32_ld, T* __restrict__ y16, int y16_ld, const float* __restrict__ u, int u_ld, int u_col,
-    const float* __restrict__ taps_w, const float* __restrict__ bias, int taps, int channels, float* __restrict__ state,
-    size_t slot_stride, size_t ring_off, const int* __restrict__ state_slots, const int* __restrict__ token_seq,
-    const int* __restrict__ positions, const int* __restrict__ cu_seqlens, const int* __restrict__ context_lens,
-    int activation, int update) {
-    const int n = blockIdx.x;
-    const int c = blockIdx.y * RC_THREADS + threadIdx.x;
-    if (c >= channels) return;
-    const int b = token_seq[n];
-    if (context_lens[b] <= 0) return;
-    const int p = positions[n];
-    const int first_row = cu_seqlens[b];
+struct ConvArgs {
+    const float* u;  // [N, u_ld], columns u_col ..
+    int u_ld, u_col;
+    const float* taps_w;  // [channels, taps]
+    const float* bias;    // [channels] or null
+    int taps, channels;
+    float* state;  // slots; the ring [taps - 1, channels] lies at ring_off inside a slot
+    size_t slot_stride, ring_off;
+    const int* state_slots;
+    const int* token_seq;
+    const int* positions;
+    const int* cu_seqlens;
+    const int* context_lens;
+    int activation, update;
+};
+
+// channel c of token n after the convolution and the activation (the token belongs to a request that exists)
+__device__ __forceinline__ float conv_channel(const ConvArgs& a, int n, int c) {
+    const int b = a.token_seq[n];
+    const int p = a.positions[n];
+    const int first_row = a.cu_seqlens[b];
     const int first_pos = p - (n - first_row);
-    float* ring = taps > 1 ? state + (size_t)state_slots[b] * slot_stride + ring_off : nullptr;
-    float y = bias ? bias[c] : 0.f;
-    for (int j = 0; j < taps; ++j) {
-        const int pos = p - (taps - 1) + j;
+    float* ring = a.taps > 1 ? a.state + (size_t)a.state_slots[b] * a.slot_stride + a.ring_off : nullptr;
+    float y = a.bias ? a.bias[c] : 0.f;
+    for (int j = 0; j < a.taps; ++j) {
+        const int pos = p - (a.taps - 1) + j;
         float v = 0.f;
         if (pos >= first_pos)
-            v = u[(size_t)(first_row + pos - first_pos) * u_ld + u_col + c];
+            v = a.u[(size_t)(first_row + pos - first_pos) * a.u_ld + a.u_col + c];
         else if (pos >= 0)
-            v = ring[(size_t)(pos % (taps - 1)) * channels + c];
-        y = fmaf(taps_w[(size_t)c * taps + j], v, y);
+            v = ring[(size_t)(pos % (a.taps - 1)) * a.channels + c];
+        y = fmaf(a.taps_w[(size_t)c * a.taps + j], v, y);
     }
-    if (update && taps > 1)  // (every request brings one token: nobody else reads this ring, and this thread has read its place)
-        ring[(size_t)(p % (taps - 1)) * channels + c] = u[(size_t)n * u_ld + u_col + c];
-    if (activation) y = rc_silu(y);
+    if (a.update && a.taps > 1)  // (every request brings one token: nobody else reads this ring, and this thread has read its place)
+        ring[(size_t)(p % (a.taps - 1)) * a.channels + c] = a.u[(size_t)n * a.u_ld + a.u_col + c];
+    return a.activation ? rc_silu(y) : y;
+}
+
+template <typename T>
+__global__ __launch_bounds__(RC_THREADS) void conv_act_kernel(float* __restrict__ y32, int y32_ld, T* __restrict__ y16, int y16_ld,
+                                                             const ConvArgs a) {
+    const int n = blockIdx.x;
+    const int c = blockIdx.y * RC_THREADS + threadIdx.x;
+    if (c >= a.channels || a.context_lens[a.token_seq[n]] <= 0) return;
+    const float y = conv_channel(a, n, c);
     if (y32) y32[(size_t)n * y32_ld + c] = y;
     if (y16) y16[(size_t)n * y16_ld + c] = from_f32<T>(y);
+}
+
+// The convolution where the first channels are heads of q and k that are made unit vectors behind it: grid (tokens, q heads
+// + k heads + blocks of 64 other channels [+ 1 for the gates]), one wave each.  A head of dk numbers (up to 256; q heads
+// first, k heads behind them, from channel 0) is divided by sqrt(sum of squares + eps), q also multiplied by q_factor; the
+// last block (with `gates`) turns the gates' products into decay and beta, as `unit_heads` does.
+#define CH_PER_LANE 4
+__global__ __launch_bounds__(LLMS_WAVE) void conv_heads_kernel(float* __restrict__ y32, int y32_ld, const ConvArgs a, int q_heads,
+                                                               int k_heads, int dk, float eps, float q_factor,
+                                                               float* __restrict__ gates, int g_ld, int a_col, int b_col,
+                                                               const float* __restrict__ a_log, const float* __restrict__ dt_bias,
+                                                               int heads) {
+    const int n = blockIdx.x, lane = threadIdx.x, role = blockIdx.y;
+    if (a.context_lens[a.token_seq[n]] <= 0) return;
+    const int first_other = (q_heads + k_heads) * dk;
+    const int other_blocks = (a.channels - first_other + LLMS_WAVE - 1) / LLMS_WAVE;
+    if (role < q_heads + k_heads) {
+        float y[CH_PER_LANE];
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < CH_PER_LANE; ++i) {
+            const int d = lane + i * LLMS_WAVE;
+            y[i] = d < dk ? conv_channel(a, n, role * dk + d) : 0.f;
+            ss = fmaf(y[i], y[i], ss);
+        }
+        const float mul = (role < q_heads ? q_factor : 1.f) / sqrtf(wave_sum(ss) + eps);
+#pragma unroll
+        for (int i = 0; i < CH_PER_LANE; ++i) {
+            const int d = lane + i * LLMS_WAVE;
+            if (d < dk) y32[(size_t)n * y32_ld + role * dk + d] = y[i] * mul;
+        }
+    } else if (role < q_heads + k_heads + other_blocks) {
+        const int c = first_other + (role - q_heads - k_heads) * LLMS_WAVE + lane;
+        if (c < a.channels) y32[(size_t)n * y32_ld + c] = conv_channel(a, n, c);
+    } else {
+        float* g = gates + (size_t)n * g_ld;
+        for (int h = lane; h < heads; h += LLMS_WAVE) {
+            g[a_col + h] = expf(-expf(a_log[h]) * rc_softplus(g[a_col + h] + dt_bias[h]));
+            g[b_col + h] = 1.f / (1.f + expf(-g[b_col + h]));
+        }
+    }
 }
 
 // grid (requests, channel blocks)
@@ -398,6 +456,17 @@ __global__ __launch_bounds__(LLMS_WAVE) void delta_finish_kernel(T* __restrict__
 
 extern "C" {
 
+static ConvArgs conv_args(const float* u, int u_ld, int u_col, const float* taps_w, const float* bias, int taps, int channels,
+                          float* state, size_t slot_stride, size_t ring_off, const int* state_slots, const int* token_seq,
+                          const int* positions, const int* cu_seqlens, const int* context_lens, int activation, int update) {
+    ConvArgs a;
+    a.u = u, a.u_ld = u_ld, a.u_col = u_col, a.taps_w = taps_w, a.bias = bias, a.taps = taps, a.channels = channels;
+    a.state = state, a.slot_stride = slot_stride, a.ring_off = ring_off, a.state_slots = state_slots;
+    a.token_seq = token_seq, a.positions = positions, a.cu_seqlens = cu_seqlens, a.context_lens = context_lens;
+    a.activation = activation, a.update = update;
+    return a;
+}
+
 int llms_conv_act(int dtype, float* y32, int y32_ld, void* y16, int y16_ld, const float* u, int u_ld, int u_col,
                   const float* taps_w, const float* bias, int taps, int channels, float* state, size_t slot_stride,
                   size_t ring_off, const int* state_slots, const int* token_seq, const int* positions, const int* cu_seqlens,
@@ -406,17 +475,36 @@ int llms_conv_act(int dtype, float* y32, int y32_ld, void* y16, int y16_ld, cons
     LLMS_REQUIRE(u && taps_w && token_seq && positions && cu_seqlens && context_lens, "conv_act: a needed operand is missing");
     LLMS_REQUIRE(taps == 1 || (state && state_slots), "conv_act: two taps or more need the state");
     LLMS_REQUIRE(y32 || y16, "conv_act: nothing to store");
+    const ConvArgs a = conv_args(u, u_ld, u_col, taps_w, bias, taps, channels, state, slot_stride, ring_off, state_slots, token_seq,
+                                 positions, cu_seqlens, context_lens, activation, update);
     dim3 grid(n_tokens, (channels + RC_THREADS - 1) / RC_THREADS);
     if (dtype == 0)
-        conv_act_kernel<float><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (float*)y16, y16_ld, u, u_ld, u_col, taps_w, bias,
-                                                                taps, channels, state, slot_stride, ring_off, state_slots,
-                                                                token_seq, positions, cu_seqlens, context_lens, activation, update);
+        conv_act_kernel<float><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (float*)y16, y16_ld, a);
     else if (dtype == 1)
-        conv_act_kernel<bf16><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (bf16*)y16, y16_ld, u, u_ld, u_col, taps_w, bias,
-                                                               taps, channels, state, slot_stride, ring_off, state_slots,
-                                                               token_seq, positions, cu_seqlens, context_lens, activation, update);
+        conv_act_kernel<bf16><<<grid, RC_THREADS, 0, stream>>>(y32, y32_ld, (bf16*)y16, y16_ld, a);
     else
         LLMS_REQUIRE(false, "conv_act: dtype must be 0 (float32) or 1 (bfloat16)");
+    LLMS_LAUNCH_CHECK();
+}
+
+int llms_conv_heads(float* y32, int y32_ld, const float* u, int u_ld, int u_col, const float* taps_w, const float* bias, int taps,
+                    int channels, float* state, size_t slot_stride, size_t ring_off, const int* state_slots, const int* token_seq,
+                    const int* positions, const int* cu_seqlens, const int* context_lens, int n_tokens, int activation, int update,
+                    int q_heads, int k_heads, int dk, float eps, float q_factor, float* gates, int g_ld, int a_col, int b_col,
+                    const float* a_log, const float* dt_bias, int heads, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && channels > 0 && taps >= 1 && y32, "conv_heads: sizes must be positive");
+    LLMS_REQUIRE(u && taps_w && token_seq && positions && cu_seqlens && context_lens, "conv_heads: a needed operand is missing");
+    LLMS_REQUIRE(taps == 1 || (state && state_slots), "conv_heads: two taps or more need the state");
+    LLMS_REQUIRE(q_heads >= 0 && k_heads >= 0 && dk > 0 && dk <= CH_PER_LANE * LLMS_WAVE && (q_heads + k_heads) * dk <= channels,
+                 "conv_heads: heads of up to 256 numbers within the channels");
+    LLMS_REQUIRE(!gates || (a_log && dt_bias && heads > 0), "conv_heads: gates need their rates and biases");
+    const ConvArgs a = conv_args(u, u_ld, u_col, taps_w, bias, taps, channels, state, slot_stride, ring_off, state_slots, token_seq,
+                                 positions, cu_seqlens, context_lens, activation, update);
+    const int blocks = q_heads + k_heads + (channels - (q_heads + k_heads) * dk + LLMS_WAVE - 1) / LLMS_WAVE + (gates ? 1 : 0);
+    LLMS_REQUIRE(blocks <= 65535, "conv_heads: too many heads and channels for one launch");
+    dim3 grid(n_tokens, blocks);
+    conv_heads_kernel<<<grid, LLMS_WAVE, 0, stream>>>(y32, y32_ld, a, q_heads, k_heads, dk, eps, q_factor, gates, g_ld, a_col, b_col,
+                                                      a_log, dt_bias, heads);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -2050,6 +2050,52 @@ def conv_act(u: torch.Tensor, u_col: int, channels: int, taps_w: torch.Tensor, *
                                   c_int(batch.num_seqs), c_int(taps), c_int(channels), _stream(dev)), "conv_ring")
 
 
+def conv_heads(u: torch.Tensor, u_col: int, channels: int, taps_w: torch.Tensor, out32: torch.Tensor, *, q_heads: int, k_heads: int,
+               dk: int, eps: float, q_factor: float = 1.0, bias: torch.Tensor | None = None, state: torch.Tensor | None = None,
+               ring_offset: int = 0, batch=None, activation: str | None = "silu", gates: dict | None = None) -> torch.Tensor:
+    """`conv_act` into out32 (float32 [N, channels]) and, in the same launch, `unit_heads` on its result: the first
+    q_heads + k_heads heads of dk channels (q first) are divided by sqrt(their sum of squares + eps), q also multiplied by
+    q_factor; `gates` as in `unit_heads`.  Heads of up to 256 numbers."""
+    dev = _dev(u, taps_w, bias, state, out32)
+    n = u.shape[0]
+    _f32_matrix(u, "u", n, u_col + channels)
+    taps = taps_w.shape[1]
+    _f32(taps_w, "taps_w", channels * taps)
+    if bias is not None:
+        _f32(bias, "bias", channels)
+    if activation not in (None, "silu"):
+        raise ValueError(f"activation {activation!r}")
+    if not 1 <= dk <= 256 or (q_heads + k_heads) * dk > channels:
+        raise ValueError("heads of 1 to 256 numbers within the channels")
+    slot_stride = _state_rows(state, batch.state_slots, (taps - 1) * channels, ring_offset, "conv_heads") if taps > 1 else 0
+    _f32_matrix(out32, "out32", n, channels)
+    for t, name in ((batch.token_seq, "token_seq"), (batch.positions, "positions")):
+        _i32(t, name, n)
+    _i32(batch.cu_seqlens, "cu_seqlens")
+    _i32(batch.context_lens, "context_lens")
+    g = gates or {}
+    if gates is not None:
+        _f32_matrix(g["gates"], "gates", n, max(g["a_col"], g["b_col"]) + g["heads"])
+        _f32(g["a_log"], "a_log", g["heads"])
+        _f32(g["dt_bias"], "dt_bias", g["heads"])
+    if n == 0:
+        return out32
+    lib = load("recurrent")
+    single = taps > 1 and batch.max_count == 1 and batch.num_seqs == n  # every request brings one token
+    _check(lib.llms_conv_heads(
+        _ptr(out32), c_int(out32.stride(0)), _ptr(u), c_int(u.stride(0)), c_int(u_col), _ptr(taps_w), _ptr(bias), c_int(taps),
+        c_int(channels), _ptr(state), c_size_t(slot_stride), c_size_t(ring_offset), _ptr(batch.state_slots), _ptr(batch.token_seq),
+        _ptr(batch.positions), _ptr(batch.cu_seqlens), _ptr(batch.context_lens), c_int(n), c_int(1 if activation == "silu" else 0),
+        c_int(1 if single else 0), c_int(q_heads), c_int(k_heads), c_int(dk), c_float(eps), c_float(q_factor), _ptr(g.get("gates")),
+        c_int(g["gates"].stride(0) if gates else 0), c_int(g.get("a_col", 0)), c_int(g.get("b_col", 0)), _ptr(g.get("a_log")),
+        _ptr(g.get("dt_bias")), c_int(g.get("heads", 0)), _stream(dev)), "conv_heads")
+    if taps > 1 and not single:
+        _check(lib.llms_conv_ring(_ptr(state), c_size_t(slot_stride), c_size_t(ring_offset), _ptr(batch.state_slots), _ptr(u),
+                                  c_int(u.stride(0)), c_int(u_col), _ptr(batch.cu_seqlens), _ptr(batch.context_lens),
+                                  c_int(batch.num_seqs), c_int(taps), c_int(channels), _stream(dev)), "conv_ring")
+    return out32
+
+
 SCAN_MAX_STATES = 256
 
 

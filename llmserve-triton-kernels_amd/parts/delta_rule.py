@@ -100,13 +100,13 @@ class GatedDelta(Mixer):
         rows, dev = x.shape[0], x.device
         proj = linear(x, self.w_in, out_dtype=torch.float32)
         qkv = torch.empty((rows, self.channels), dtype=torch.float32, device=dev)
-        ops.conv_act(proj, 0, self.channels, self.taps_w, state=cache.state, ring_offset=self.scan_numbers, batch=batch,
-                     out32=qkv)
         gates = dict(gates=proj, a_col=self.col_a, b_col=self.col_b, a_log=self.a_log, dt_bias=self.dt_bias, heads=self.heads)
         # (steps of many tokens: decay and beta are formed beside the recurrence, not inside its chain from token to token)
         many = batch.max_count > self.PREPARE_FROM
-        ops.unit_heads(qkv, q_col=0, k_col=self.cq, q_heads=self.kv_heads, k_heads=self.kv_heads, dk=self.dk,
-                       eps=self.unit_eps, q_factor=self.dk ** -0.5, gates=gates if many else None)
+        # the convolution, SiLU, the unit vectors (and the gates) in one launch
+        ops.conv_heads(proj, 0, self.channels, self.taps_w, qkv, q_heads=self.kv_heads, k_heads=self.kv_heads, dk=self.dk,
+                       eps=self.unit_eps, q_factor=self.dk ** -0.5, state=cache.state, ring_offset=self.scan_numbers, batch=batch,
+                       gates=gates if many else None)
         o = torch.empty((rows, self.cv), dtype=torch.float32, device=dev)
         ops.delta_scan(o, qkv, q_col=0, k_col=self.cq, v_col=2 * self.cq, kv_heads=self.kv_heads, dk=self.dk, dv=self.dv,
                        state=cache.state, scan_offset=0, batch=batch, prepared=many, **gates)

@@ -28,7 +28,6 @@ from __future__ import annotations
 import torch
 
 from ..ops import library as ops
-from .linear import linear
 from .registry import FeedForward, register_feed_forward
 from .spec import ParamInfo
 
@@ -68,7 +67,16 @@ class Experts(FeedForward):
         self.shared_gated = bool(shared.get("gate", False)) if shared else False
         if shared and self.shared_intermediate < 1:
             raise ValueError("the shared unit needs a positive width")
-        self.w_shared_gate_up = self.w_shared_down = self.b_router = None
+        self.b_router = None
+        self.shared_unit = None  # the shared expert: the engine's dense gated feed-forward under its own tensor names
+        if shared:
+            from .registry import FEED_FORWARDS
+            from .spec import PartSpec
+
+            n = self.names
+            self.shared_unit = FEED_FORWARDS.build(PartSpec("swiglu", {
+                "hidden": self.hidden, "intermediate": self.shared_intermediate, "result": "float32",
+                "names": {"gate": n["shared_gate"], "up": n["shared_up"], "down": n["shared_down"]}}), ctx)
         if not 1 <= self.top <= min(self.experts, ops.MOE_MAX_TOP):
             raise ValueError(f"top={self.top} of {self.experts} experts (at most {ops.MOE_MAX_TOP})")
         self.w_router = self.w_gate_up = self.w_down = None
@@ -85,10 +93,8 @@ class Experts(FeedForward):
             infos[n["down"].format(e=e)] = ParamInfo((h, i))
         if self.router_bias:
             infos[n["router_bias"]] = ParamInfo((self.experts,), "around_zero")
-        if self.shared_intermediate:
-            s = self.shared_intermediate
-            infos[n["shared_gate"]], infos[n["shared_up"]] = ParamInfo((s, h)), ParamInfo((s, h))
-            infos[n["shared_down"]] = ParamInfo((h, s))
+        if self.shared_unit is not None:
+            infos.update(self.shared_unit.param_infos())
             if self.shared_gated:
                 infos[n["shared_sg"]] = ParamInfo((1, h))
         return infos
@@ -98,9 +104,8 @@ class Experts(FeedForward):
         self.w_router = tensors[n["router"]].contiguous()
         if self.router_bias:
             self.b_router = tensors[n["router_bias"]].float().contiguous()
-        if self.shared_intermediate:
-            self.w_shared_gate_up = torch.cat([tensors[n["shared_gate"]], tensors[n["shared_up"]]], dim=0).contiguous()
-            self.w_shared_down = tensors[n["shared_down"]].contiguous()
+        if self.shared_unit is not None:
+            self.shared_unit.load({name: tensors[name] for name in self.shared_unit.param_infos()})
             if self.shared_gated:  # the gate's row lies behind the experts' in the router's matrix: one kernel forms both
                 self.w_router = torch.cat([self.w_router, tensors[n["shared_sg"]].reshape(1, self.hidden)], dim=0).contiguous()
         # [E, 64 ceil(I / 32), H]: blocks of 32 gate rows and the 32 up rows of the same units, so that a thread of
@@ -118,11 +123,7 @@ class Experts(FeedForward):
         ops.moe_router(chosen, weight, x, self.w_router, renormalize=self.renormalize, scores=self.scores,
                        groups=self.groups, keep=self.keep, renorm_eps=self.renorm_eps, bias=self.b_router,
                        extra_out=shared_gate)
-        shared = None
-        if self.shared_intermediate:
-            unit = torch.empty((rows, self.shared_intermediate), dtype=x.dtype, device=dev)
-            ops.silu_mul(unit, linear(x, self.w_shared_gate_up))
-            shared = linear(unit, self.w_shared_down, out_dtype=torch.float32)
+        shared = self.shared_unit.forward(x) if self.shared_unit is not None else None
         on_input = self.weight_on == "input"
         sorted_in = torch.empty((pairs, self.hidden), dtype=x.dtype, device=dev)
         place = torch.empty(pairs, dtype=torch.int32, device=dev)

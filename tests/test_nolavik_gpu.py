@@ -210,7 +210,7 @@ def delta_weights(width, heads, kv, dk, dv, taps, seed):
             "norm": rnd(dv, seed=seed + 11) + 1.0, "o": torch.eye(heads * dv, dtype=F64)}
 
 
-def run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, portions):
+def run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, portions, fused=True):
     from llmserve.ops import library as ops
 
     t = h.shape[0]
@@ -226,11 +226,16 @@ def run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, portions):
         batch = step_of([n], [a + n], [2])
         proj = dev(proj_all[a: a + n])
         qkv = torch.empty((n, channels), dtype=torch.float32, device=DEV)
-        ops.conv_act(proj, 0, channels, taps_w, state=state, ring_offset=scan, batch=batch, out32=qkv)
         gates = dict(gates=proj, a_col=channels + cv, b_col=channels + cv + heads, a_log=dev(w["A_log"]), dt_bias=dev(w["dt_bias"]),
                      heads=heads)
         many = n > 2  # (decay and beta formed beside the recurrence, as the part does for portions of several tokens)
-        ops.unit_heads(qkv, q_col=0, k_col=cq, q_heads=kv, k_heads=kv, dk=dk, eps=1e-6, q_factor=dk ** -0.5, gates=gates if many else None)
+        if fused:  # the convolution, the unit vectors and the gates in one launch, as the part does
+            ops.conv_heads(proj, 0, channels, taps_w, qkv, q_heads=kv, k_heads=kv, dk=dk, eps=1e-6, q_factor=dk ** -0.5, state=state,
+                           ring_offset=scan, batch=batch, gates=gates if many else None)
+        else:
+            ops.conv_act(proj, 0, channels, taps_w, state=state, ring_offset=scan, batch=batch, out32=qkv)
+            ops.unit_heads(qkv, q_col=0, k_col=cq, q_heads=kv, k_heads=kv, dk=dk, eps=1e-6, q_factor=dk ** -0.5,
+                           gates=gates if many else None)
         o = torch.full((n, cv), float("nan"), dtype=torch.float32, device=DEV)
         ops.delta_scan(o, qkv, q_col=0, k_col=cq, v_col=2 * cq, kv_heads=kv, dk=dk, dv=dv, state=state, scan_offset=0, batch=batch,
                        prepared=many, **gates)
@@ -248,7 +253,12 @@ def test_the_delta_rule_whole_and_in_portions(heads, kv, dk, dv, taps, dtype):
     h, w = rnd(t, width, seed=40), delta_weights(width, heads, kv, dk, dv, taps, seed=41)
     want = pn.gated_delta(h, w, "", {"heads": heads, "kv_heads": kv, "dim": dk, "vdim": dv, "conv": taps}, eps)
     close(run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, (1000,)), want, dtype, "whole", loose=3)
-    close(run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, (7, 2, 1, 19, 1, 1)), want, dtype, "in portions", loose=3)
+    in_portions_fused = run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, (7, 2, 1, 19, 1, 1))
+    close(in_portions_fused, want, dtype, "in portions", loose=3)
+    # the kernels the fused launch stands for give the same numbers
+    in_portions_apart = run_delta(h, w, heads, kv, dk, dv, taps, eps, dtype, (7, 2, 1, 19, 1, 1), fused=False)
+    close(in_portions_apart, want, dtype, "in portions, convolution and unit vectors apart", loose=3)
+    assert (in_portions_apart.double() - in_portions_fused.double()).abs().max() <= 1e-5 * float(want.abs().max())
 
 
 def test_the_read_out_sees_the_tokens_own_write():
