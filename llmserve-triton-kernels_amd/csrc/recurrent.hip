@@ -8,12 +8,13 @@
 //                   because a token's write would race with its neighbours' reads; when every request brings one
 //                   token, conv_act writes the ring itself).
 //   selective_scan  per channel c and state n:  S <- exp(dt_c A[c, n]) S + dt_c x_c B_n,  y_c = sum_n S C_n + D_c x_c,
-//                   dt = softplus(dt_raw + bias), and y silu(z) leaves rounded once.  16 lanes share a channel's states.
+//                   dt from `step_sizes`, and y silu(z) leaves rounded once.  16 lanes share a channel's states.
 //   conv_heads      conv_act and unit_heads in one launch, a wave a head: what the delta rule's layer runs.
 //   unit_heads      every head of q and k is divided by sqrt(sum of squares + eps); q is multiplied by a factor; where
 //                   a step brings many tokens it also turns the gates' products into decay and beta, and
-//   scan_prepare    forms the step sizes and silu(z) of the selective scan, so that no logarithm and no exponential
-//                   besides the recurrence's own stands in the chain from token to token.
+//   step_sizes      forms the step sizes (their small product, the bias, softplus) and, for steps of many tokens, silu(z)
+//                   of the selective scan, so that no logarithm and no exponential besides the recurrence's own stands
+//                   in the chain from token to token.
 //   delta_scan      the gated delta rule per head over a state S [dk, dv]:
 //                   S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q   (the read-out sees the token's write)
 //                   with beta = sigmoid(zb) and g = exp(-exp(A_log) softplus(za + dt_bias)).  16 lanes share a column.
@@ -162,8 +163,8 @@ __global__ __launch_bounds__(RC_THREADS) void conv_ring_kernel(
 // grid (requests, channels / 16).  Thread (channel, lane of 16): states lane, lane + 16, ...  R = ceil(states / 16).
 // x [N, x_ld] (after the convolution), z [N, z_ld] columns z_col .., low [N, low_ld]: B at b_col, C at c_col,
 // dt_raw [N, dt_ld]; S [channels, states] at scan_off inside a slot.
-// PREP: dt_raw already holds softplus(dt_raw + bias) and z already silu(z) (`scan_prepare`), which keeps the
-// logarithm and the exponentials that do not belong to the recurrence out of its chain.
+// dt holds the step sizes (`step_sizes`).  PREP: z already holds silu(z) (the same launch), which keeps the exponential
+// that does not belong to the recurrence out of its chain.
 template <typename T, int R, bool PREP>
 __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
     T* __restrict__ out, int out_ld, const float* __restrict__ x, int x_ld, const float* __restrict__ z, int z_ld, int z_col,
@@ -186,7 +187,7 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
         s[r] = k < states ? srow[k] : 0.f;
         a[r] = k < states ? a_neg[(size_t)cc * states + k] : 0.f;
     }
-    const float bias = dt_bias[cc], skip = d_skip[cc];
+    const float skip = d_skip[cc];
     // tokens in groups of U, two groups in registers: the next group is asked for before the present one is worked on, so
     // the chain from token to token never waits for memory
     constexpr int U = R <= 2 ? 8 : (R <= 4 ? 4 : 2);
@@ -216,7 +217,7 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             if (t0 + u >= count) break;
-            const float dt = PREP ? g.dtr[u] : rc_softplus(g.dtr[u] + bias);
+            const float dt = g.dtr[u];
             const float dx = dt * g.xs[u];
             float y = 0.f;
 #pragma unroll
@@ -263,14 +264,50 @@ __global__ __launch_bounds__(RC_THREADS) void selective_scan_kernel(
     }
 }
 
-// grid (tokens, channel blocks): dt_raw <- softplus(dt_raw + bias), z <- silu(z), in place
-__global__ __launch_bounds__(RC_THREADS) void scan_prepare_kernel(float* __restrict__ dt_raw, int dt_ld, const float* __restrict__ dt_bias,
-                                                                 float* __restrict__ z, int z_ld, int z_col, int channels) {
-    const int n = blockIdx.x, c = blockIdx.y * RC_THREADS + threadIdx.x;
+// grid (blocks of SS_TOKENS tokens, blocks of 64 channels): dt[n, c] = softplus(sum_r low[n, low_col + r] w_t[r, c] + bias[c]),
+// the step sizes' product (a weight of few columns, kept transposed so that neighbouring threads read neighbouring
+// numbers; a number of the weight serves SS_TOKENS tokens) with what follows it; with `z`, z <- silu(z) in place as well
+#define SS_TOKENS 8
+__global__ __launch_bounds__(LLMS_WAVE) void step_sizes_kernel(float* __restrict__ dt, int dt_ld, const float* __restrict__ low,
+                                                               int low_ld, int low_col, int rank, const float* __restrict__ w_t,
+                                                               const float* __restrict__ dt_bias, float* __restrict__ z, int z_ld,
+                                                               int z_col, int channels, int n_tokens) {
+    extern __shared__ float lows[];  // [rank][SS_TOKENS]
+    const int n0 = blockIdx.x * SS_TOKENS, c = blockIdx.y * LLMS_WAVE + threadIdx.x;
+    for (int i = threadIdx.x; i < rank * SS_TOKENS; i += LLMS_WAVE) {
+        const int t = i % SS_TOKENS, r = i / SS_TOKENS;
+        lows[i] = n0 + t < n_tokens ? low[(size_t)(n0 + t) * low_ld + low_col + r] : 0.f;
+    }
+    __syncthreads();
     if (c >= channels) return;
-    dt_raw[(size_t)n * dt_ld + c] = rc_softplus(dt_raw[(size_t)n * dt_ld + c] + dt_bias[c]);
-    float* zp = z + (size_t)n * z_ld + z_col + c;
-    *zp = rc_silu(*zp);
+    float acc[SS_TOKENS];
+#pragma unroll
+    for (int t = 0; t < SS_TOKENS; ++t) acc[t] = 0.f;
+    int r = 0;
+    for (; r + 16 <= rank; r += 16) {  // sixteen numbers of the weight asked for at once (few waves run when decoding)
+        float w[16];
+#pragma unroll
+        for (int k = 0; k < 16; ++k) w[k] = w_t[(size_t)(r + k) * channels + c];
+#pragma unroll
+        for (int k = 0; k < 16; ++k)
+#pragma unroll
+            for (int t = 0; t < SS_TOKENS; ++t) acc[t] = fmaf(lows[(r + k) * SS_TOKENS + t], w[k], acc[t]);
+    }
+    for (; r < rank; ++r) {
+        const float w = w_t[(size_t)r * channels + c];
+#pragma unroll
+        for (int t = 0; t < SS_TOKENS; ++t) acc[t] = fmaf(lows[r * SS_TOKENS + t], w, acc[t]);
+    }
+    const float bias = dt_bias[c];
+#pragma unroll
+    for (int t = 0; t < SS_TOKENS; ++t) {
+        if (n0 + t >= n_tokens) break;
+        dt[(size_t)(n0 + t) * dt_ld + c] = rc_softplus(acc[t] + bias);
+        if (z) {
+            float* zp = z + (size_t)(n0 + t) * z_ld + z_col + c;
+            *zp = rc_silu(*zp);
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------- unit heads
@@ -561,11 +598,13 @@ int llms_unit_heads(float* x, int ld, int q_col, int k_col, int q_heads, int k_h
     LLMS_LAUNCH_CHECK();
 }
 
-int llms_scan_prepare(float* dt_raw, int dt_ld, const float* dt_bias, float* z, int z_ld, int z_col, int channels, int n_tokens,
-                      hipStream_t stream) {
-    LLMS_REQUIRE(n_tokens > 0 && channels > 0, "scan_prepare: sizes must be positive");
-    dim3 grid(n_tokens, (channels + RC_THREADS - 1) / RC_THREADS);
-    scan_prepare_kernel<<<grid, RC_THREADS, 0, stream>>>(dt_raw, dt_ld, dt_bias, z, z_ld, z_col, channels);
+int llms_step_sizes(float* dt, int dt_ld, const float* low, int low_ld, int low_col, int rank, const float* w_t,
+                    const float* dt_bias, float* z, int z_ld, int z_col, int channels, int n_tokens, hipStream_t stream) {
+    LLMS_REQUIRE(n_tokens > 0 && channels > 0 && rank > 0 && rank <= 1024, "step_sizes: sizes must be positive, up to 1,024 columns");
+    LLMS_REQUIRE((channels + LLMS_WAVE - 1) / LLMS_WAVE <= 65535, "step_sizes: too many channels for one launch");
+    dim3 grid((n_tokens + SS_TOKENS - 1) / SS_TOKENS, (channels + LLMS_WAVE - 1) / LLMS_WAVE);
+    step_sizes_kernel<<<grid, LLMS_WAVE, (size_t)rank * SS_TOKENS * sizeof(float), stream>>>(dt, dt_ld, low, low_ld, low_col, rank, w_t,
+                                                                                          dt_bias, z, z_ld, z_col, channels, n_tokens);
     LLMS_LAUNCH_CHECK();
 }
 

@@ -2099,17 +2099,38 @@ def conv_heads(u: torch.Tensor, u_col: int, channels: int, taps_w: torch.Tensor,
 SCAN_MAX_STATES = 256
 
 
+def step_sizes(dt: torch.Tensor, low: torch.Tensor, low_col: int, w_t: torch.Tensor, bias: torch.Tensor, *,
+               z: torch.Tensor | None = None, z_col: int = 0) -> torch.Tensor:
+    """dt[n, c] = softplus(sum_r low[n, low_col + r] w_t[r, c] + bias[c]), all 32-bit: low float32 [N, >=], w_t float32
+    [rank, channels] (the weight transposed), dt float32 [N, channels].  With `z` (float32 [N, >= z_col + channels]) the same
+    launch turns z's columns into silu(z), in place."""
+    dev = _dev(dt, low, w_t, bias, z)
+    n, channels = dt.shape
+    if w_t.dim() != 2 or w_t.shape[1] != channels:
+        raise ValueError("w_t is [rank, channels]")
+    rank = w_t.shape[0]
+    _f32(w_t, "w_t", rank * channels)
+    _f32(bias, "bias", channels)
+    _f32_matrix(dt, "dt", n, channels)
+    _f32_matrix(low, "low", n, low_col + rank)
+    if z is not None:
+        _f32_matrix(z, "z", n, z_col + channels)
+    if n:
+        _check(load("recurrent").llms_step_sizes(
+            _ptr(dt), c_int(dt.stride(0)), _ptr(low), c_int(low.stride(0)), c_int(low_col), c_int(rank), _ptr(w_t), _ptr(bias),
+            _ptr(z), c_int(z.stride(0) if z is not None else 0), c_int(z_col), c_int(channels), c_int(n), _stream(dev)), "step_sizes")
+    return dt
+
+
 def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: int, low: torch.Tensor, b_col: int, c_col: int,
-                   dt_raw: torch.Tensor, dt_bias: torch.Tensor, a_neg: torch.Tensor, d_skip: torch.Tensor,
-                   state: torch.Tensor, scan_offset: int, batch, prepare: bool = False) -> torch.Tensor:
+                   dt: torch.Tensor, a_neg: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, scan_offset: int, batch,
+                   z_prepared: bool = False) -> torch.Tensor:
     """Per request, token by token, per channel c and state n:  S[c, n] <- exp(dt_c a_neg[c, n]) S[c, n] + dt_c x_c B_n,
-    y_c = sum_n S[c, n] C_n + d_skip[c] x_c, with dt = softplus(dt_raw + dt_bias); out[t, c] = y_c silu(z_c), rounded
-    once.  x float32 [N, channels]; z float32 [N, >= z_col + channels]; low float32 [N, >=] with B at b_col and C at
-    c_col (`states` numbers each); dt_raw float32 [N, channels]; S float32 [channels, states] at `scan_offset` of the
-    request's slot of `state`, read before the first token and left behind the last.  `prepare`: a launch of its own
-    first turns dt_raw into the step sizes and z into silu(z), in place (for steps of many tokens: the recurrence is a
-    chain from token to token, and what does not depend on it is better done beside it)."""
-    dev = _dev(out, x, z, low, dt_raw, dt_bias, a_neg, d_skip, state)
+    y_c = sum_n S[c, n] C_n + d_skip[c] x_c; out[t, c] = y_c silu(z_c), rounded once.  x float32 [N, channels]; z float32
+    [N, >= z_col + channels] (`z_prepared`: it already holds silu(z), see `step_sizes`); low float32 [N, >=] with B at
+    b_col and C at c_col (`states` numbers each); dt float32 [N, channels], the step sizes; S float32 [channels, states]
+    at `scan_offset` of the request's slot of `state`, read before the first token and left behind the last."""
+    dev = _dev(out, x, z, low, dt, a_neg, d_skip, state)
     n, channels = x.shape
     if a_neg.dim() != 2 or a_neg.shape[0] != channels:
         raise ValueError("a_neg is [channels, states]")
@@ -2119,8 +2140,7 @@ def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: i
     _f32_matrix(x, "x", n, channels)
     _f32_matrix(z, "z", n, z_col + channels)
     _f32_matrix(low, "low", n, max(b_col, c_col) + states)
-    _f32_matrix(dt_raw, "dt_raw", n, channels)
-    _f32(dt_bias, "dt_bias", channels)
+    _f32_matrix(dt, "dt", n, channels)
     _f32(a_neg, "a_neg", channels * states)
     _f32(d_skip, "d_skip", channels)
     if out.dim() != 2 or out.stride(1) != 1 or out.shape != (n, channels):
@@ -2130,15 +2150,12 @@ def selective_scan(out: torch.Tensor, x: torch.Tensor, z: torch.Tensor, z_col: i
     _i32(batch.context_lens, "context_lens")
     if n == 0:
         return out
-    if prepare:
-        _check(load("recurrent").llms_scan_prepare(_ptr(dt_raw), c_int(dt_raw.stride(0)), _ptr(dt_bias), _ptr(z), c_int(z.stride(0)),
-                                                   c_int(z_col), c_int(channels), c_int(n), _stream(dev)), "scan_prepare")
     _check(load("recurrent").llms_selective_scan(
         c_int(_code(out)), _ptr(out), c_int(out.stride(0)), _ptr(x), c_int(x.stride(0)), _ptr(z), c_int(z.stride(0)),
-        c_int(z_col), _ptr(low), c_int(low.stride(0)), c_int(b_col), c_int(c_col), _ptr(dt_raw), c_int(dt_raw.stride(0)),
-        _ptr(dt_bias), _ptr(a_neg), _ptr(d_skip), c_int(channels), c_int(states), _ptr(state), c_size_t(slot_stride),
+        c_int(z_col), _ptr(low), c_int(low.stride(0)), c_int(b_col), c_int(c_col), _ptr(dt), c_int(dt.stride(0)),
+        _ptr(None), _ptr(a_neg), _ptr(d_skip), c_int(channels), c_int(states), _ptr(state), c_size_t(slot_stride),
         c_size_t(scan_offset), _ptr(batch.state_slots), _ptr(batch.cu_seqlens), _ptr(batch.context_lens),
-        c_int(batch.num_seqs), c_int(1 if prepare else 0), _stream(dev)), "selective_scan")
+        c_int(batch.num_seqs), c_int(1 if z_prepared else 0), _stream(dev)), "selective_scan")
     return out
 
 

@@ -50,7 +50,7 @@ def _fill_skip(shape, generator, device, options):
 @register_mixer("selective_scan")
 class SelectiveScan(Mixer):
     graph_safe = True
-    PREPARE_FROM = 4  # new tokens of the longest portion beyond which step sizes and gate get a launch of their own
+    PREPARE_FROM = 4  # new tokens of the longest portion beyond which silu(z) is formed beside the recurrence
 
     def __init__(self, spec, ctx):
         super().__init__(spec, ctx)
@@ -64,7 +64,7 @@ class SelectiveScan(Mixer):
         if min(self.hidden, self.inner, self.dt_rank, self.taps) < 1 or not 1 <= self.states <= ops.SCAN_MAX_STATES:
             raise ValueError(f"sizes must be positive, with 1 to {ops.SCAN_MAX_STATES} states per channel")
         self.scan_numbers = self.inner * self.states  # S first, then the ring
-        self.w_in = self.w_x = self.w_dt = self.w_o = self.taps_w = self.conv_bias = self.dt_bias = self.a_neg = self.skip = None
+        self.w_in = self.w_x = self.w_dt_t = self.w_o = self.taps_w = self.conv_bias = self.dt_bias = self.a_neg = self.skip = None
 
     def libraries(self, dtype_name):
         return ("recurrent",)
@@ -84,7 +84,7 @@ class SelectiveScan(Mixer):
         n = self.names
         self.w_in = tensors[n["in"]].contiguous()
         self.w_x = tensors[n["x"]].contiguous()
-        self.w_dt = tensors[n["dt"]].float().contiguous()
+        self.w_dt_t = tensors[n["dt"]].float().t().contiguous()  # [dt_rank, inner]
         self.w_o = tensors[n["o"]].contiguous()
         self.taps_w = tensors[n["conv"]].float().contiguous()
         self.conv_bias = tensors[n["conv_bias"]].float().contiguous()
@@ -100,9 +100,12 @@ class SelectiveScan(Mixer):
         ops.conv_act(xz, 0, c, self.taps_w, bias=self.conv_bias, state=cache.state, ring_offset=self.scan_numbers,
                      batch=batch, out32=x32, out16=None if x16 is x32 else x16)
         low = linear(x16, self.w_x, out_dtype=torch.float32)
-        # (the step sizes' product is small and stays 32-bit whatever the model's dtype: its input is not rounded)
-        dt_raw = ops.gemm_fma(torch.empty((rows, c), dtype=torch.float32, device=dev), low[:, :self.dt_rank], self.w_dt)
+        # the step sizes' product is small and stays 32-bit whatever the model's dtype (its input is not rounded): one kernel
+        # with the bias and softplus; with many tokens it also forms silu(z), which then stands beside the recurrence's chain
+        many = batch.max_count > self.PREPARE_FROM
+        dt = ops.step_sizes(torch.empty((rows, c), dtype=torch.float32, device=dev), low, 0, self.w_dt_t, self.dt_bias,
+                            z=xz if many else None, z_col=c)
         out = torch.empty((rows, c), dtype=x.dtype, device=dev)
-        ops.selective_scan(out, x32, xz, c, low, self.dt_rank, self.dt_rank + self.states, dt_raw, self.dt_bias, self.a_neg,
-                           self.skip, cache.state, 0, batch, prepare=batch.max_count > self.PREPARE_FROM)
+        ops.selective_scan(out, x32, xz, c, low, self.dt_rank, self.dt_rank + self.states, dt, self.a_neg, self.skip, cache.state,
+                           0, batch, z_prepared=many)
         return linear(out, self.w_o, out_dtype=self.result_dtype)

@@ -163,11 +163,13 @@ def test_the_selective_scan_whole_and_in_portions(inner, states, rank, taps, dty
             ops.conv_act(proj, 0, inner, dev(w["conv"]), bias=dev(w["conv.b"]), state=state, ring_offset=inner * states, batch=batch,
                          out32=x32)
             low = dev(x32.double().cpu() @ w["x"].T)
-            dt_raw = dev(low.double().cpu()[:, :rank] @ w["dt"].T)
+            many = n > 2  # (portions of several tokens: silu(z) formed beside the recurrence, as the part does)
+            dt = ops.step_sizes(torch.empty((n, inner), dtype=torch.float32, device=DEV), low, 0, dev(w["dt"].T), dev(w["dt.b"]),
+                                z=proj if many else None, z_col=inner)
+            close(dt, pn.softplus(low.double().cpu()[:, :rank] @ w["dt"].T + w["dt.b"]), torch.float32, "step sizes", loose=3)
             out = torch.full((n, inner), float("nan"), dtype=dtype, device=DEV)
-            # (portions of several tokens: step sizes and gate formed by a launch of their own, as the part does)
-            ops.selective_scan(out, x32, proj, inner, low, rank, rank + states, dt_raw, dev(w["dt.b"]), dev(-torch.exp(w["A_log"])),
-                               dev(w["D"]), state, 0, batch, prepare=n > 2)
+            ops.selective_scan(out, x32, proj, inner, low, rank, rank + states, dt, dev(-torch.exp(w["A_log"])), dev(w["D"]), state, 0,
+                               batch, z_prepared=many)
             outs.append(out.cpu())
         close(torch.cat(outs), want, dtype, f"portions {portions}", loose=3)
         assert bool(torch.isnan(state[0]).all()) and bool(torch.isnan(state[2]).all())
@@ -184,18 +186,17 @@ def test_a_scan_whose_state_must_last():
     low = torch.zeros(t, 2 * states, dtype=F64)
     low[0, :states] = 1.0          # B of the first token
     low[t - 1, states:] = 1.0      # C of the last
-    dt_raw = torch.full((t, inner), 0.5413, dtype=F64)  # softplus -> about 1
+    dt = 1.25
+    steps = torch.full((t, inner), dt, dtype=F64)
     a_neg = torch.full((inner, states), -1e-4, dtype=F64)
-    dt = float(pn.softplus(torch.tensor(0.5413, dtype=F64)))
     want_last = states * dt * 5.0 * math.exp(-1e-4 * dt * (t - 1))
     state = torch.zeros((1, inner * states), dtype=torch.float32, device=DEV)
     z = torch.full((t, inner), 30.0, dtype=F64)  # silu(30) = 30
     last = None
     for a, n in in_portions(t, (64, 1, 1, 130, 2)):
         out = torch.empty((n, inner), dtype=torch.float32, device=DEV)
-        ops.selective_scan(out, dev(x[a: a + n]), dev(z[a: a + n]), 0, dev(low[a: a + n]), 0, states, dev(dt_raw[a: a + n]),
-                           dev(torch.zeros(inner, dtype=F64)), dev(a_neg), dev(torch.zeros(inner, dtype=F64)), state, 0,
-                           step_of([n], [a + n], [0]))
+        ops.selective_scan(out, dev(x[a: a + n]), dev(z[a: a + n]), 0, dev(low[a: a + n]), 0, states, dev(steps[a: a + n]),
+                           dev(a_neg), dev(torch.zeros(inner, dtype=F64)), state, 0, step_of([n], [a + n], [0]))
         last = out[-1].cpu()
     assert float(last[0]) == pytest.approx(30.0 * want_last, rel=1e-4)
 
